@@ -33,14 +33,24 @@ class Config:
     dist_init_method: str = "tcp://127.0.0.1:2333"
     dist_backend: Optional[str] = None  # None: "nccl" (RCCL) on GPUs, "gloo" on CPU
     direct_all_reduce: bool = True    # TP > 1 on GPUs: decode-sized all-reduces over IPC-mapped peer buffers (lv_comm)
+    dtype: Optional[str] = None       # "bfloat16" | "float32": overrides the checkpoint's dtype (f32: models whose kernels have it)
+    max_cache_tokens: int = -1        # ragged-step models: > 0 sizes the page pool for this many tokens instead of from free HBM
+    long_prefill_token_threshold: int = 0   # ragged-step models: > 0 caps the prompt tokens one sequence gets per step
 
     def __post_init__(self):
-        assert self.kvcache_block_size % 256 == 0, "kvcache_block_size must be a multiple of 256"
         assert 1 <= self.tensor_parallel_size <= 8
         assert self.device == "cpu" or self.device == "cuda" or self.device.startswith("cuda:")
         if self.hf_config is None:
             assert self.model is not None and os.path.isdir(self.model), f"'{self.model}' is not a model directory"
-            from transformers import AutoConfig
-            self.hf_config = AutoConfig.from_pretrained(self.model)
+            from .models.registry import load_config
+            self.hf_config = load_config(self.model)
+        from .models.registry import model_class
+        self.ragged = bool(getattr(model_class(self.hf_config), "ragged_steps", False))
+        if not self.ragged:     # the paged softmax-attention kernels walk the cache in 256-token pages
+            assert self.kvcache_block_size % 256 == 0, "kvcache_block_size must be a multiple of 256"
+        if self.dtype is not None:
+            import torch
+            self.hf_config.torch_dtype = {"bfloat16": torch.bfloat16, "float32": torch.float32}[self.dtype]
+            assert self.ragged or self.dtype == "bfloat16", "this model's attention kernels are bf16 only"
         self.max_model_len = min(self.max_model_len, self.hf_config.max_position_embeddings)
-        assert self.max_num_batched_tokens >= self.max_model_len
+        assert self.ragged or self.max_num_batched_tokens >= self.max_model_len

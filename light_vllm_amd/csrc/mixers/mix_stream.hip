@@ -1,0 +1,451 @@
+// Residual-stream kernels and the gated delta rule.
+//
+//   hc_update_norm_kernel     one workgroup per token: the S residual streams are remixed and receive the
+//                             sublayer output, and in the same pass the next sublayer's input is read out
+//                             of them and normalised in groups. Streams and all arithmetic are f32.
+//   clamped_glu_kernel        elementwise gate of the feed-forward.
+//   delta_prep_kernel         one wave per (token, head slot): convolution taps from the step's own rows
+//                             or the carried state, silu, unit norm; one more wave per token for the
+//                             write strength and the decay.
+//   conv_state_update_kernel  one thread per (sequence, channel) shifts the carried inputs.
+//   gated_delta_rule_kernel   one workgroup per (64 value columns, head, sequence) walks the step's tokens;
+//                             each lane owns one column of the state, the four waves own a quarter of the
+//                             rows each, partial dot products meet in LDS once per token.
+//   head_norm_gate_kernel     one wave per (token, head).
+#include "mix_common.h"
+
+namespace lvmix {
+
+static thread_local char g_err[512] = "";
+
+int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+int launched(const char* what) {
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(-3, "%s: launch failed: %s", what, hipGetErrorString(e));
+  return 0;
+}
+
+// ------------------------------------------------------------------------------------------------
+template <typename T, int S>
+__global__ __launch_bounds__(256) void hc_update_norm_kernel(float* __restrict__ x, const T* __restrict__ y,
+                                                              const float* __restrict__ mix,
+                                                              const float* __restrict__ out_w,
+                                                              const float* __restrict__ in_w,
+                                                              const float* __restrict__ norm_w, T* __restrict__ out,
+                                                              int W, int groups, float eps) {
+  extern __shared__ float lds[];          // [W] read-out, then [groups] inverse rms
+  float* u_lds = lds;
+  float* inv_lds = lds + W;
+  const int64_t t = blockIdx.x;
+  float* xt = x + t * S * W;
+  float m[S][S], ow[S], iw[S];
+#pragma unroll
+  for (int s = 0; s < S; ++s) {
+    ow[s] = y != nullptr ? out_w[s] : 0.0f;
+    iw[s] = out != nullptr ? in_w[s] : 0.0f;
+#pragma unroll
+    for (int r = 0; r < S; ++r) m[s][r] = y != nullptr ? mix[s * S + r] : 0.0f;
+  }
+  for (int i = threadIdx.x; i < W; i += blockDim.x) {
+    float xs[S];
+#pragma unroll
+    for (int s = 0; s < S; ++s) xs[s] = xt[s * W + i];
+    if (y != nullptr) {
+      const float yv = ldf(y + t * W + i);
+      float nx[S];
+#pragma unroll
+      for (int r = 0; r < S; ++r) {
+        float acc = ow[r] * yv;
+#pragma unroll
+        for (int s = 0; s < S; ++s) acc += m[s][r] * xs[s];
+        nx[r] = acc;
+      }
+#pragma unroll
+      for (int s = 0; s < S; ++s) {
+        xs[s] = nx[s];
+        xt[s * W + i] = nx[s];
+      }
+    }
+    if (out != nullptr) {
+      float u = 0.0f;
+#pragma unroll
+      for (int s = 0; s < S; ++s) u += iw[s] * xs[s];
+      u_lds[i] = u;
+    }
+  }
+  if (out == nullptr) return;
+  __syncthreads();
+  const int gs = W / groups;
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave, nwaves = blockDim.x / kWave;
+  for (int g = wave; g < groups; g += nwaves) {
+    float ss = 0.0f;
+    for (int i = lane; i < gs; i += kWave) {
+      const float v = u_lds[g * gs + i];
+      ss += v * v;
+    }
+    ss = wave_sum(ss);
+    if (lane == 0) inv_lds[g] = 1.0f / sqrtf(ss / static_cast<float>(gs) + eps);
+  }
+  __syncthreads();
+  for (int i = threadIdx.x; i < W; i += blockDim.x)
+    stf(out + t * W + i, u_lds[i] * inv_lds[i / gs] * norm_w[i]);
+}
+
+template <typename T>
+static int hc_launch(void* x, const void* y, const void* mix, const void* out_w, const void* in_w,
+                     const void* norm_w, void* out, int64_t Tn, int S, int W, int groups, float eps,
+                     hipStream_t stream) {
+  const size_t shm = static_cast<size_t>(W + groups) * sizeof(float);
+  dim3 grid(static_cast<unsigned>(Tn)), block(256);
+#define LVMIX_HC(SS)                                                                                            \
+  case SS:                                                                                                      \
+    hc_update_norm_kernel<T, SS><<<grid, block, shm, stream>>>(                                                 \
+        static_cast<float*>(x), static_cast<const T*>(y), static_cast<const float*>(mix),                       \
+        static_cast<const float*>(out_w), static_cast<const float*>(in_w), static_cast<const float*>(norm_w),   \
+        static_cast<T*>(out), W, groups, eps);                                                                  \
+    break;
+  switch (S) {
+    LVMIX_HC(1) LVMIX_HC(2) LVMIX_HC(3) LVMIX_HC(4) LVMIX_HC(5) LVMIX_HC(6) LVMIX_HC(7) LVMIX_HC(8)
+    default: return fail(-2, "lv_hc_update_norm: %d streams (1..%d supported)", S, LV_MIX_MAX_STREAMS);
+  }
+#undef LVMIX_HC
+  return launched("lv_hc_update_norm");
+}
+
+// ------------------------------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void clamped_glu_kernel(const T* __restrict__ in, int64_t ld_in, T* __restrict__ out,
+                                                          int64_t Tn, int F, float limit, float alpha) {
+  const int64_t idx = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (idx >= Tn * F) return;
+  const int64_t t = idx / F;
+  const int f = static_cast<int>(idx - t * F);
+  const float g = fminf(ldf(in + t * ld_in + f), limit);
+  const float u = fminf(fmaxf(ldf(in + t * ld_in + F + f), -limit), limit);
+  stf(out + idx, g * sigmoidf_(alpha * g) * (u + 1.0f));
+}
+
+// ------------------------------------------------------------------------------------------------
+struct DeltaPrepParams {
+  const void* proj;
+  int64_t ld;
+  const float* conv_w;
+  const void* conv_state;
+  const float* A_log;
+  const float* dt_bias;
+  const int32_t *cu_q, *ctx_lens, *slots, *tok_seq;
+  float *qn, *kn, *v, *beta, *decay;
+  int64_t T;
+  int G, H, D, Dv, taps, off_b, off_a;
+  float unit_eps;
+};
+
+template <typename T>
+__global__ __launch_bounds__(256) void delta_prep_kernel(DeltaPrepParams p) {
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+  const int64_t t = blockIdx.x;
+  const int unit = blockIdx.y * (blockDim.x / kWave) + wave;
+  const int units = 2 * p.G + p.H + 1;
+  if (unit >= units) return;
+  const T* proj = static_cast<const T*>(p.proj);
+  const int b = p.tok_seq[t];
+  const int q0 = p.cu_q[b];
+  const int r = static_cast<int>(t) - q0;         // index of the token inside its sequence's portion
+  const int ctx = p.ctx_lens[b];
+  if (unit == units - 1) {                        // write strength and decay, one lane per head
+    for (int h = lane; h < p.H; h += kWave) {
+      const float bv = ldf(proj + t * p.ld + p.off_b + h);
+      const float av = ldf(proj + t * p.ld + p.off_a + h);
+      p.beta[t * p.H + h] = sigmoidf_(bv);
+      p.decay[t * p.H + h] = expf(-expf(p.A_log[h]) * softplusf_(av + p.dt_bias[h]));
+    }
+    return;
+  }
+  const int C = 2 * p.G * p.D + p.H * p.Dv;
+  const int taps = p.taps;
+  const T* state = static_cast<const T*>(p.conv_state) + static_cast<int64_t>(p.slots[b]) * (taps - 1) * C;
+  int c0, n;
+  float* dst;
+  bool unit_norm = true;
+  float post = 1.0f;
+  if (unit < p.G) {
+    c0 = unit * p.D; n = p.D; dst = p.qn + (t * p.G + unit) * p.D; post = 1.0f / sqrtf(static_cast<float>(p.D));
+  } else if (unit < 2 * p.G) {
+    c0 = p.G * p.D + (unit - p.G) * p.D; n = p.D; dst = p.kn + (t * p.G + (unit - p.G)) * p.D;
+  } else {
+    const int h = unit - 2 * p.G;
+    c0 = 2 * p.G * p.D + h * p.Dv; n = p.Dv; dst = p.v + (t * p.H + h) * p.Dv; unit_norm = false;
+  }
+  float ss = 0.0f;
+  for (int e = lane; e < n; e += kWave) {
+    const int c = c0 + e;
+    float acc = 0.0f;
+    for (int i = 0; i < taps; ++i) {
+      const int rr = r - (taps - 1 - i);          // row of the portion this tap reads
+      float xin = 0.0f;
+      if (rr >= 0) xin = ldf(proj + static_cast<int64_t>(q0 + rr) * p.ld + c);
+      else if (ctx + rr >= 0) xin = ldf(state + static_cast<int64_t>(taps - 1 + rr) * C + c);
+      acc += p.conv_w[c * taps + i] * xin;
+    }
+    const float a = siluf_(acc);
+    dst[e] = a;
+    ss += a * a;
+  }
+  if (!unit_norm) return;
+  ss = wave_sum(ss);
+  const float inv = post / sqrtf(ss + p.unit_eps);
+  for (int e = lane; e < n; e += kWave) dst[e] *= inv;    // each lane rescales what it wrote itself
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void conv_state_update_kernel(const T* __restrict__ proj, int64_t ld,
+                                                                T* __restrict__ conv_state,
+                                                                const int32_t* __restrict__ cu_q,
+                                                                const int32_t* __restrict__ ctx_lens,
+                                                                const int32_t* __restrict__ slots, int C, int taps) {
+  const int b = blockIdx.y;
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  if (c >= C) return;
+  const int q0 = cu_q[b], n = cu_q[b + 1] - q0, ctx = ctx_lens[b];
+  if (n <= 0) return;
+  T* state = conv_state + static_cast<int64_t>(slots[b]) * (taps - 1) * C;
+  // new row s holds the input of position ctx + n - (taps-1) + s; ascending s reads old rows above s only
+  for (int s = 0; s < taps - 1; ++s) {
+    const int rr = n - (taps - 1) + s;
+    float v = 0.0f;
+    if (rr >= 0) v = ldf(proj + static_cast<int64_t>(q0 + rr) * ld + c);
+    else if (ctx + rr >= 0) v = ldf(state + static_cast<int64_t>(taps - 1 + rr) * C + c);
+    stf(state + static_cast<int64_t>(s) * C + c, v);
+  }
+}
+
+// ------------------------------------------------------------------------------------------------
+struct DeltaRuleParams {
+  const float *qn, *kn, *v, *beta, *decay;
+  float* state;
+  const int32_t *cu_q, *ctx_lens, *slots;
+  float* o;
+  int G, H, D, Dv;
+};
+
+// DR = rows of the state each of the four waves owns (4 * DR >= D; rows beyond D stay zero).
+template <int DR>
+__global__ __launch_bounds__(256) void gated_delta_rule_kernel(DeltaRuleParams p) {
+  __shared__ float part_k[2][4][kWave];
+  __shared__ float part_o[2][4][kWave];
+  const int lane = threadIdx.x % kWave, rp = threadIdx.x / kWave;
+  const int col = blockIdx.x * kWave + lane;
+  const int h = blockIdx.y, b = blockIdx.z;
+  const int g = h / (p.H / p.G);
+  const int q0 = p.cu_q[b], n = p.cu_q[b + 1] - q0;
+  if (n <= 0) return;
+  const bool live = col < p.Dv;
+  const int row0 = rp * DR;
+  float* sbase = p.state + (static_cast<int64_t>(p.slots[b]) * p.H + h) * p.D * p.Dv;
+  float s[DR];
+  const bool carry = p.ctx_lens[b] > 0;
+#pragma unroll
+  for (int r = 0; r < DR; ++r)
+    s[r] = (carry && live && row0 + r < p.D) ? sbase[static_cast<int64_t>(row0 + r) * p.Dv + col] : 0.0f;
+
+  for (int i = 0; i < n; ++i) {
+    const int64_t t = q0 + i;
+    const int buf = i & 1;
+    const float* kt = p.kn + (t * p.G + g) * p.D;
+    const float* qt = p.qn + (t * p.G + g) * p.D;
+    float kr[DR], qr[DR];
+#pragma unroll
+    for (int r = 0; r < DR; ++r) {
+      const bool in = row0 + r < p.D;
+      kr[r] = in ? kt[row0 + r] : 0.0f;
+      qr[r] = in ? qt[row0 + r] : 0.0f;
+    }
+    const float beta = p.beta[t * p.H + h];
+    const float dec = p.decay[t * p.H + h];
+    const float vv = live ? p.v[(t * p.H + h) * p.Dv + col] : 0.0f;
+    float pk = 0.0f;
+#pragma unroll
+    for (int r = 0; r < DR; ++r) pk += s[r] * kr[r];
+    part_k[buf][rp][lane] = pk;
+    __syncthreads();
+    // the previous token's read-out partials are complete behind this barrier as well
+    if (i > 0 && rp == ((i - 1) & 3) && live) {
+      const int pb = buf ^ 1;
+      p.o[((t - 1) * p.H + h) * p.Dv + col] = part_o[pb][0][lane] + part_o[pb][1][lane] + part_o[pb][2][lane] + part_o[pb][3][lane];
+    }
+    const float ks = part_k[buf][0][lane] + part_k[buf][1][lane] + part_k[buf][2][lane] + part_k[buf][3][lane];
+    const float u = beta * (vv - dec * ks);         // the state is decayed before it is read
+    float po = 0.0f;
+#pragma unroll
+    for (int r = 0; r < DR; ++r) {
+      s[r] = dec * s[r] + kr[r] * u;
+      po += s[r] * qr[r];
+    }
+    part_o[buf][rp][lane] = po;
+  }
+  __syncthreads();
+  {
+    const int pb = (n - 1) & 1;
+    if (rp == 0 && live)
+      p.o[((static_cast<int64_t>(q0) + n - 1) * p.H + h) * p.Dv + col] =
+          part_o[pb][0][lane] + part_o[pb][1][lane] + part_o[pb][2][lane] + part_o[pb][3][lane];
+  }
+  if (live) {
+#pragma unroll
+    for (int r = 0; r < DR; ++r)
+      if (row0 + r < p.D) sbase[static_cast<int64_t>(row0 + r) * p.Dv + col] = s[r];
+  }
+}
+
+// ------------------------------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void head_norm_gate_kernel(const float* __restrict__ o, const T* __restrict__ gate,
+                                                             int64_t ld_gate, const float* __restrict__ norm_w,
+                                                             T* __restrict__ out, int64_t items, int H, int Dv,
+                                                             float eps) {
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+  const int64_t item = static_cast<int64_t>(blockIdx.x) * (blockDim.x / kWave) + wave;   // (token, head)
+  if (item >= items) return;
+  const int64_t t = item / H;
+  const int h = static_cast<int>(item - t * H);
+  const float* row = o + item * Dv;
+  float ss = 0.0f;
+  for (int e = lane; e < Dv; e += kWave) ss += row[e] * row[e];
+  ss = wave_sum(ss);
+  const float inv = 1.0f / sqrtf(ss / static_cast<float>(Dv) + eps);
+  for (int e = lane; e < Dv; e += kWave) {
+    const float gv = ldf(gate + t * ld_gate + h * Dv + e);
+    stf(out + item * Dv + e, row[e] * inv * norm_w[e] * siluf_(gv));
+  }
+}
+
+}  // namespace lvmix
+
+using namespace lvmix;
+
+extern "C" {
+
+int lv_mix_abi_version(void) { return LV_MIX_ABI_VERSION; }
+const char* lv_mix_last_error(void) { return lvmix::g_err; }
+
+int lv_hc_update_norm(void* x, const void* y, const void* mix, const void* out_w, const void* in_w,
+                      const void* norm_w, void* out, int64_t T, int S, int W, int groups, float eps, int dtype,
+                      void* stream) {
+  if (T == 0) return 0;
+  if (x == nullptr || T < 0 || W <= 0) return fail(-1, "lv_hc_update_norm: bad arguments");
+  if (y != nullptr && (mix == nullptr || out_w == nullptr)) return fail(-1, "lv_hc_update_norm: y without mix/out_w");
+  if (out != nullptr && (in_w == nullptr || norm_w == nullptr || groups <= 0 || W % groups != 0))
+    return fail(-1, "lv_hc_update_norm: read-out needs in_w, norm_w and groups dividing W (%d, %d)", W, groups);
+  if (static_cast<size_t>(W + groups) * 4 > 160 * 1024) return fail(-2, "lv_hc_update_norm: width %d too large", W);
+  if (dtype == LV_MIX_BF16)
+    return hc_launch<bf16_t>(x, y, mix, out_w, in_w, norm_w, out, T, S, W, groups > 0 ? groups : 1, eps, as_stream(stream));
+  if (dtype == LV_MIX_F32)
+    return hc_launch<float>(x, y, mix, out_w, in_w, norm_w, out, T, S, W, groups > 0 ? groups : 1, eps, as_stream(stream));
+  return fail(-1, "lv_hc_update_norm: dtype %d", dtype);
+}
+
+int lv_clamped_glu(const void* in, int64_t ld_in, void* out, int64_t T, int F, float limit, float alpha, int dtype,
+                   void* stream) {
+  if (T == 0) return 0;
+  if (in == nullptr || out == nullptr || T < 0 || F <= 0 || ld_in < 2 * F) return fail(-1, "lv_clamped_glu: bad arguments");
+  const int64_t n = T * F;
+  dim3 grid(static_cast<unsigned>((n + 255) / 256)), block(256);
+  if (dtype == LV_MIX_BF16)
+    clamped_glu_kernel<bf16_t><<<grid, block, 0, as_stream(stream)>>>(static_cast<const bf16_t*>(in), ld_in,
+                                                                    static_cast<bf16_t*>(out), T, F, limit, alpha);
+  else if (dtype == LV_MIX_F32)
+    clamped_glu_kernel<float><<<grid, block, 0, as_stream(stream)>>>(static_cast<const float*>(in), ld_in,
+                                                                   static_cast<float*>(out), T, F, limit, alpha);
+  else
+    return fail(-1, "lv_clamped_glu: dtype %d", dtype);
+  return launched("lv_clamped_glu");
+}
+
+int lv_delta_prep(const void* proj, int64_t ld, const void* conv_w, const void* conv_state, const void* A_log,
+                  const void* dt_bias, const int32_t* cu_q, const int32_t* ctx_lens, const int32_t* slots,
+                  const int32_t* tok_seq, void* qn, void* kn, void* v, void* beta, void* decay, int64_t T, int G,
+                  int H, int D, int Dv, int taps, int off_b, int off_a, float unit_eps, int dtype, void* stream) {
+  if (T == 0) return 0;
+  if (!proj || !conv_w || !conv_state || !A_log || !dt_bias || !cu_q || !ctx_lens || !slots || !tok_seq || !qn ||
+      !kn || !v || !beta || !decay)
+    return fail(-1, "lv_delta_prep: null pointer");
+  if (G <= 0 || H <= 0 || H % G != 0 || D <= 0 || Dv <= 0 || taps < 1) return fail(-1, "lv_delta_prep: bad sizes");
+  const int C = 2 * G * D + H * Dv;
+  if (ld < C || off_b + H > ld || off_a + H > ld) return fail(-1, "lv_delta_prep: row stride %lld too small", (long long)ld);
+  DeltaPrepParams p{proj, ld, static_cast<const float*>(conv_w), conv_state, static_cast<const float*>(A_log),
+                    static_cast<const float*>(dt_bias), cu_q, ctx_lens, slots, tok_seq, static_cast<float*>(qn),
+                    static_cast<float*>(kn), static_cast<float*>(v), static_cast<float*>(beta),
+                    static_cast<float*>(decay), T, G, H, D, Dv, taps, off_b, off_a, unit_eps};
+  const int units = 2 * G + H + 1;
+  dim3 grid(static_cast<unsigned>(T), (units + 3) / 4), block(256);
+  if (dtype == LV_MIX_BF16) delta_prep_kernel<bf16_t><<<grid, block, 0, as_stream(stream)>>>(p);
+  else if (dtype == LV_MIX_F32) delta_prep_kernel<float><<<grid, block, 0, as_stream(stream)>>>(p);
+  else return fail(-1, "lv_delta_prep: dtype %d", dtype);
+  return launched("lv_delta_prep");
+}
+
+int lv_conv_state_update(const void* proj, int64_t ld, void* conv_state, const int32_t* cu_q, const int32_t* ctx_lens,
+                         const int32_t* slots, int B, int C, int taps, int dtype, void* stream) {
+  if (B == 0 || taps <= 1) return 0;
+  if (!proj || !conv_state || !cu_q || !ctx_lens || !slots || B < 0 || C <= 0 || ld < C)
+    return fail(-1, "lv_conv_state_update: bad arguments");
+  dim3 grid((C + 255) / 256, B), block(256);
+  if (dtype == LV_MIX_BF16)
+    conv_state_update_kernel<bf16_t><<<grid, block, 0, as_stream(stream)>>>(
+        static_cast<const bf16_t*>(proj), ld, static_cast<bf16_t*>(conv_state), cu_q, ctx_lens, slots, C, taps);
+  else if (dtype == LV_MIX_F32)
+    conv_state_update_kernel<float><<<grid, block, 0, as_stream(stream)>>>(
+        static_cast<const float*>(proj), ld, static_cast<float*>(conv_state), cu_q, ctx_lens, slots, C, taps);
+  else
+    return fail(-1, "lv_conv_state_update: dtype %d", dtype);
+  return launched("lv_conv_state_update");
+}
+
+int lv_gated_delta_rule(const void* qn, const void* kn, const void* v, const void* beta, const void* decay, void* state,
+                        const int32_t* cu_q, const int32_t* ctx_lens, const int32_t* slots, void* o, int B, int G,
+                        int H, int D, int Dv, void* stream) {
+  if (B == 0) return 0;
+  if (!qn || !kn || !v || !beta || !decay || !state || !cu_q || !ctx_lens || !slots || !o)
+    return fail(-1, "lv_gated_delta_rule: null pointer");
+  if (B < 0 || G <= 0 || H <= 0 || H % G != 0 || D <= 0 || Dv <= 0) return fail(-1, "lv_gated_delta_rule: bad sizes");
+  if (D > 256) return fail(-2, "lv_gated_delta_rule: key size %d above 256", D);
+  DeltaRuleParams p{static_cast<const float*>(qn), static_cast<const float*>(kn), static_cast<const float*>(v),
+                    static_cast<const float*>(beta), static_cast<const float*>(decay), static_cast<float*>(state),
+                    cu_q, ctx_lens, slots, static_cast<float*>(o), G, H, D, Dv};
+  dim3 grid((Dv + kWave - 1) / kWave, H, B), block(256);
+  hipStream_t s = as_stream(stream);
+  if (D <= 32) gated_delta_rule_kernel<8><<<grid, block, 0, s>>>(p);
+  else if (D <= 64) gated_delta_rule_kernel<16><<<grid, block, 0, s>>>(p);
+  else if (D <= 128) gated_delta_rule_kernel<32><<<grid, block, 0, s>>>(p);
+  else gated_delta_rule_kernel<64><<<grid, block, 0, s>>>(p);
+  return launched("lv_gated_delta_rule");
+}
+
+int lv_head_norm_gate(const void* o, const void* gate, int64_t ld_gate, const void* norm_w, void* out, int64_t T,
+                      int H, int Dv, float eps, int dtype, void* stream) {
+  if (T == 0) return 0;
+  if (!o || !gate || !norm_w || !out || T < 0 || H <= 0 || Dv <= 0 || ld_gate < static_cast<int64_t>(H) * Dv)
+    return fail(-1, "lv_head_norm_gate: bad arguments");
+  const int64_t items = T * H;
+  dim3 grid(static_cast<unsigned>((items + 3) / 4)), block(256);
+  if (dtype == LV_MIX_BF16)
+    head_norm_gate_kernel<bf16_t><<<grid, block, 0, as_stream(stream)>>>(
+        static_cast<const float*>(o), static_cast<const bf16_t*>(gate), ld_gate, static_cast<const float*>(norm_w),
+        static_cast<bf16_t*>(out), items, H, Dv, eps);
+  else if (dtype == LV_MIX_F32)
+    head_norm_gate_kernel<float><<<grid, block, 0, as_stream(stream)>>>(
+        static_cast<const float*>(o), static_cast<const float*>(gate), ld_gate, static_cast<const float*>(norm_w),
+        static_cast<float*>(out), items, H, Dv, eps);
+  else
+    return fail(-1, "lv_head_norm_gate: dtype %d", dtype);
+  return launched("lv_head_norm_gate");
+}
+
+}  // extern "C"

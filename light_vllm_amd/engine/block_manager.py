@@ -130,6 +130,16 @@ class BlockManager:
         seq.num_cached_tokens = 0
         seq.block_table.clear()
 
+    # -- page-by-page growth without the prefix cache: for models whose sequences also carry state
+    #    that pages do not hold (a cached prefix could not be resumed), and for portions of prompts
+    def can_extend(self, seq: Sequence, num_tokens: int) -> bool:
+        return len(self._free) >= -(-num_tokens // self.block_size) - len(seq.block_table)
+
+    def extend(self, seq: Sequence, num_tokens: int) -> None:
+        """Pages for the first `num_tokens` tokens of the sequence; taken pages are never hashed."""
+        while len(seq.block_table) * self.block_size < num_tokens:
+            seq.block_table.append(self._take_head().block_id)
+
     def can_append(self, seq: Sequence) -> bool:
         boundary = 0 if self.strict_reference else 1
         needs_new_block = len(seq) % self.block_size == boundary

@@ -35,7 +35,9 @@ class LLMEngine:
             self.events.append(event)
         self.model_runner = ModelRunner(config, 0, self.events)
         self.tokenizer = None
-        if config.model is not None:
+        import os
+        if config.model is not None and any(os.path.exists(os.path.join(config.model, f))
+                                            for f in ("tokenizer.json", "tokenizer_config.json", "tokenizer.model")):
             from transformers import AutoTokenizer
             self.tokenizer = AutoTokenizer.from_pretrained(config.model, use_fast=True)
             config.eos = self.tokenizer.eos_token_id
@@ -62,10 +64,15 @@ class LLMEngine:
     def step(self):
         seqs, is_prefill = self.scheduler.schedule()
         all_greedy = all(seq.temperature == 0 for seq in seqs)
+        if self.config.ragged:
+            scheduled = [seq.num_scheduled_tokens for seq in seqs]      # read before postprocess clears them
         token_ids = self.model_runner.call("run", seqs, is_prefill, all_greedy)
         self.scheduler.postprocess(seqs, token_ids)
         outputs = [(seq.seq_id, seq.completion_token_ids) for seq in seqs if seq.is_finished]
-        num_tokens = sum(len(seq) for seq in seqs) if is_prefill else -len(seqs)
+        if self.config.ragged:
+            num_tokens = sum(scheduled) if is_prefill else -len(seqs)
+        else:
+            num_tokens = sum(len(seq) for seq in seqs) if is_prefill else -len(seqs)
         return outputs, num_tokens
 
     def is_finished(self):

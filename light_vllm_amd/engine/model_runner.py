@@ -32,8 +32,8 @@ import torch.distributed as dist
 from .. import ops
 from ..config import Config
 from ..layers.sampler import Sampler
-from ..models.qwen3 import Qwen3ForCausalLM
-from ..utils.context import get_context, reset_context, set_context
+from ..models.registry import model_class
+from ..utils.context import RaggedStep, get_context, reset_context, set_context
 from ..utils.loader import load_model, load_random, load_random_on_device
 from .sequence import Sequence
 
@@ -52,7 +52,10 @@ class ModelRunner:
         self.block_size = config.kvcache_block_size
         self.max_position = hf_config.max_position_embeddings
         Sequence.set_block_size(self.block_size)
-        self.enforce_eager = config.enforce_eager
+        # ragged-step models (recurrent / windowed mixers): one eager code path for prompts, portions and
+        # decoded tokens; their kernels come from liblvmix.so and the paged-attention library stays unloaded
+        self.ragged = bool(getattr(config, "ragged", False))
+        self.enforce_eager = config.enforce_eager or self.ragged
         self.world_size = config.tensor_parallel_size
         self.rank = rank
         self.event = event
@@ -86,7 +89,10 @@ class ModelRunner:
         torch.set_default_dtype(dtype)
         torch.set_default_device(self.device)
         try:
-            self.model = Qwen3ForCausalLM(hf_config)
+            if dtype == torch.float32:
+                torch.backends.cuda.matmul.allow_tf32 = False      # f32 means f32 in the GEMMs as well
+                torch.backends.cudnn.allow_tf32 = False
+            self.model = model_class(hf_config)(hf_config)
             if config.random_seed is not None and config.random_on_device:
                 load_random_on_device(self.model, config.random_seed)
             elif config.random_seed is not None:
@@ -97,9 +103,12 @@ class ModelRunner:
             self.kv_cache = None
             if self.world_size > 1:
                 dist.barrier()          # every rank has its weights: the first collective starts together
-            self.warmup_model()
-            self.reserve_workspace()
-            self.allocate_kv_cache()
+            if self.ragged:
+                self.allocate_ragged_cache()
+            else:
+                self.warmup_model()
+                self.reserve_workspace()
+                self.allocate_kv_cache()
             if not self.enforce_eager:
                 self.capture_graphs()
         finally:
@@ -269,6 +278,36 @@ class ModelRunner:
                 layer_id += 1
         assert layer_id == hf.num_hidden_layers
 
+    def allocate_ragged_cache(self) -> None:
+        """Pages and state slots of a ragged-step model. Every mixer module states what a page and a
+        slot cost it (`cache_bytes`) and allocates its own tensors (`bind_cache`); all of them share
+        the page ids of one block table and the slot ids of the state manager. The pool is sized for
+        `max_cache_tokens` when given, else from free device memory after a reserve for the
+        activations of the largest step."""
+        cfg = self.config
+        act_bytes = torch.empty((), dtype=self.dtype).element_size()
+        users = [m for m in self.model.modules() if hasattr(m, "cache_bytes") and hasattr(m, "bind_cache")]
+        per_block = sum(m.cache_bytes(self.block_size, act_bytes)[0] for m in users)
+        per_slot = sum(m.cache_bytes(self.block_size, act_bytes)[1] for m in users)
+        num_slots = cfg.max_num_seqs
+        if cfg.max_cache_tokens > 0:
+            num_blocks = -(-cfg.max_cache_tokens // self.block_size)
+        elif cfg.num_kvcache_blocks > 0:
+            num_blocks = cfg.num_kvcache_blocks
+        else:
+            assert self.on_gpu, "CPU plumbing runs need max_cache_tokens or num_kvcache_blocks"
+            free, total = torch.cuda.mem_get_info()
+            hf = cfg.hf_config
+            reserve = cfg.max_num_batched_tokens * hf.hidden_size * (8 * getattr(hf, "streams", 1) + 64)
+            available = int(total * cfg.gpu_memory_utilization) - (total - free) - reserve - per_slot * num_slots
+            num_blocks = available // max(per_block, 1) if per_block else 1
+            num_blocks = min(num_blocks, num_slots * -(-cfg.max_model_len // self.block_size))
+        assert num_blocks > 0, "not enough memory for the cache"
+        cfg.num_kvcache_blocks = int(num_blocks)
+        self.cache_sizing = dict(per_block=per_block, per_slot=per_slot, blocks=int(num_blocks), slots=num_slots)
+        for m in users:
+            m.bind_cache(int(num_blocks), self.block_size, num_slots, self.device, self.dtype)
+
     # ------------------------------------------------------------------ step inputs
     def _check_positions(self, last_position: int) -> None:
         """Positions index the rotary table (max_position_embeddings rows). The fused kernel clamps
@@ -376,6 +415,63 @@ class ModelRunner:
         return build_plan(lens + [0] * (bucket - bs), hkv, hq // hkv, max_splits=self.plan_row_splits(),
                           capacity=bucket + self.plan_extra_items)
 
+    def prepare_ragged(self, seqs: list[Sequence], rows=None):
+        """Step inputs of a ragged batch: sequence b brings its next `num_scheduled_tokens` tokens
+        behind the `num_computed_tokens` it already has in the cache and its state slot. `rows`: packed
+        token indices whose logits are wanted (None: the last token of every sequence)."""
+        input_ids, positions, tok_seq = [], [], []
+        cu_q, ctx_lens, slots, lens_q = [0], [], [], []
+        for b, seq in enumerate(seqs):
+            n, ctx = seq.num_scheduled_tokens, seq.num_computed_tokens
+            assert n > 0 and ctx + n <= len(seq) and seq.state_slot >= 0
+            assert len(seq.block_table) * self.block_size >= ctx + n, "sequence lacks pages for its new tokens"
+            input_ids.extend(seq[ctx:ctx + n])
+            positions.extend(range(ctx, ctx + n))
+            tok_seq.extend([b] * n)
+            cu_q.append(cu_q[-1] + n)
+            ctx_lens.append(ctx)
+            lens_q.append(n)
+            slots.append(seq.state_slot)
+        if rows is None:
+            rows = [c - 1 for c in cu_q[1:]]
+        tables = [list(seq.block_table) for seq in seqs]
+        step = RaggedStep(self._to_device(cu_q, torch.int32), self._to_device(ctx_lens, torch.int32),
+                          self._to_device(slots, torch.int32), self._to_device(tok_seq, torch.int32),
+                          self.prepare_block_tables(seqs), lens_q, ctx_lens, slots, tables)
+        set_context(any(n > 1 for n in lens_q), ragged=step, logits_indices=self._to_device(rows, torch.int64))
+        return self._to_device(input_ids, torch.int64), self._to_device(positions, torch.int64)
+
+    @torch.inference_mode()
+    def run_rows(self, seqs: list[Sequence], rows: list[int]):
+        """One ragged step; returns the f32 logits [len(rows), vocab] of the packed token rows `rows` on
+        the host (an empty tensor when no row is wanted: the step still advances cache and state)."""
+        input_ids, positions = self.prepare_ragged(seqs, rows)
+        hidden = self.model(input_ids, positions)
+        logits = self.model.compute_logits(hidden).float().cpu() if rows else torch.empty(0, 0)
+        reset_context()
+        return logits
+
+    @torch.inference_mode()
+    def run_ragged(self, seqs: list[Sequence], all_greedy: bool):
+        """A scheduled ragged step: a token for every sequence whose known tokens end with this step,
+        None for those that are still in the middle of their prompt."""
+        done = [seq.num_computed_tokens + seq.num_scheduled_tokens == len(seq) for seq in seqs]
+        ends, at = [], 0
+        for seq in seqs:
+            at += seq.num_scheduled_tokens
+            ends.append(at - 1)
+        rows = [r for r, d in zip(ends, done) if d]
+        input_ids, positions = self.prepare_ragged(seqs, rows)
+        hidden = self.model(input_ids, positions)
+        tokens = []
+        if rows:
+            logits = self.model.compute_logits(hidden)
+            temperatures = self.prepare_sample([seq for seq, d in zip(seqs, done) if d])
+            tokens = self.sampler(logits, temperatures, all_greedy).tolist()
+        reset_context()
+        it = iter(tokens)
+        return [next(it) if d else None for d in done]
+
     def prepare_sample(self, seqs: list[Sequence]) -> torch.Tensor:
         return self._to_device([seq.temperature for seq in seqs], torch.float32)
 
@@ -432,6 +528,8 @@ class ModelRunner:
         instead of gathering [batch, vocab] logits to rank 0 (ParallelLMHead.greedy_tokens): the
         same token, 16 bytes per sequence and rank on the wire instead of 2 * vocab / tp."""
         self._check_direct_comm()       # ranks that never sync see the steps before this one here
+        if getattr(self, "ragged", False):
+            return self.run_ragged(seqs, all_greedy)
         input_ids, positions = self.prepare_prefill(seqs) if is_prefill else self.prepare_decode(seqs)
         if all_greedy and self.world_size > 1:
             tokens = self.run_model(input_ids, positions, is_prefill, greedy=True)

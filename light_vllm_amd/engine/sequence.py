@@ -45,6 +45,11 @@ class Sequence:
         # True until the sequence's KV is in the cache: at creation and again after a preemption
         # (the scheduler sets it). Decides what the step RPC ships to the workers, see __getstate__.
         self.needs_prefill = True
+        # ragged-step models: tokens whose K/V and state the engine holds, tokens the current step
+        # computes, and the slot of the state manager (-1: none)
+        self.num_computed_tokens = 0
+        self.num_scheduled_tokens = 0
+        self.state_slot = -1
 
     def __len__(self) -> int:
         return self.num_tokens
@@ -91,6 +96,13 @@ class Sequence:
     def get_token_ids_from_block(self, i: int) -> list[int]:
         assert 0 <= i < self.num_blocks
         return self.token_ids[i * self.block_size:(i + 1) * self.block_size]
+
+    def extend_tokens(self, token_ids: list[int]) -> None:
+        """More known tokens for a sequence that is fed piecewise (a prompt that arrives in portions)."""
+        self.token_ids.extend(token_ids)
+        self.last_token = self.token_ids[-1]
+        self.num_tokens = len(self.token_ids)
+        self.num_prompt_tokens = self.num_tokens
 
     def append_token(self, token_id: int) -> None:
         self.token_ids.append(token_id)

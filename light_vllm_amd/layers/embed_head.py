@@ -60,7 +60,9 @@ class ParallelLMHead(VocabParallelEmbedding):
 
     def forward(self, x: torch.Tensor):
         context = get_context()
-        if context.is_prefill:
+        if context.logits_indices is not None:
+            x = x[context.logits_indices].contiguous()
+        elif context.is_prefill:
             last_indices = context.cu_seqlens_q[1:] - 1
             x = x[last_indices].contiguous()
         logits = F.linear(x, self.weight, self.bias)
@@ -78,7 +80,9 @@ class ParallelLMHead(VocabParallelEmbedding):
         gathers to rank 0 (layers/embed_head.py:175-195) - here every rank ends up with it.
         For steps whose sequences are all greedy; one rank: plain argmax."""
         context = get_context()
-        if context.is_prefill:
+        if context.logits_indices is not None:
+            x = x[context.logits_indices].contiguous()
+        elif context.is_prefill:
             last_indices = context.cu_seqlens_q[1:] - 1
             x = x[last_indices].contiguous()
         logits = F.linear(x, self.weight, self.bias).float()

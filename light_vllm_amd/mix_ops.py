@@ -1,0 +1,309 @@
+"""Tensor-level wrappers over liblvmix.so (include/lv_mixers.h), one function per kernel.
+
+GPU tensors go to the HIP kernels (bf16 or f32 activations; streams, recurrent state and the small
+parameter vectors always f32). CPU tensors, which only the plumbing tests of the engine produce,
+take a restatement in torch ops ON THE SAME cache and state layouts, so that page tables, state
+slots and ragged batching are exercised without a GPU. Nothing here synchronises.
+
+`step` is the utils.context.RaggedStep of the running forward pass: device tensors cu_q [B+1],
+ctx_lens [B], slots [B], tok_seq [T], block_tables [B, n] and the same lengths as python ints.
+"""
+from __future__ import annotations
+
+import math
+
+import torch
+import torch.nn.functional as F
+
+from . import _mixlib
+
+_DT = {torch.bfloat16: 0, torch.float32: 1}
+
+
+def _stream(t: torch.Tensor) -> int:
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def _p(t):
+    return None if t is None else t.data_ptr()
+
+
+def _f32(*ts):
+    for t in ts:
+        assert t is None or (t.dtype == torch.float32 and t.is_contiguous()), "expected a contiguous f32 tensor"
+
+
+# ---------------------------------------------------------------------------------------- streams
+def hc_update_norm(x, y=None, mix=None, out_w=None, in_w=None, norm_w=None, groups=1, eps=1e-6, act_dtype=None):
+    """x [T, S, W] f32 is updated in place from the sublayer output y [T, W] (skipped when y is None);
+    returns the grouped-RMS-normed read-out sum_s in_w[s] x[s] in act dtype (None when in_w is None)."""
+    T, S, W = x.shape
+    _f32(x, mix, out_w, in_w, norm_w)
+    act_dtype = act_dtype or (y.dtype if y is not None else torch.bfloat16)
+    out = torch.empty(T, W, dtype=act_dtype, device=x.device) if in_w is not None else None
+    if x.is_cuda:
+        if y is not None:
+            assert y.is_contiguous() and y.dtype == act_dtype and y.shape == (T, W)
+        lib = _mixlib.load()
+        _mixlib.check(lib.lv_hc_update_norm(_p(x), _p(y), _p(mix), _p(out_w), _p(in_w), _p(norm_w), _p(out), T, S, W,
+                                            groups, eps, _DT[act_dtype], _stream(x)), "lv_hc_update_norm")
+        return out
+    if y is not None:
+        x.copy_(torch.einsum("sr,tsw->trw", mix, x) + out_w[None, :, None] * y.float()[:, None, :])
+    if in_w is None:
+        return None
+    u = torch.einsum("s,tsw->tw", in_w, x)
+    ug = u.view(T, groups, W // groups)
+    ug = ug / torch.sqrt(ug.pow(2).mean(-1, keepdim=True) + eps)
+    out.copy_(ug.reshape(T, W) * norm_w)
+    return out
+
+
+def clamped_glu(x, limit: float, alpha: float):
+    """x [T, 2F] = [gate | up] -> min(g, L) * sigmoid(alpha * g) * (clamp(u, -L, L) + 1), [T, F]."""
+    T, F2 = x.shape
+    Fh = F2 // 2
+    out = torch.empty(T, Fh, dtype=x.dtype, device=x.device)
+    if x.is_cuda:
+        assert x.stride(1) == 1
+        lib = _mixlib.load()
+        _mixlib.check(lib.lv_clamped_glu(_p(x), x.stride(0), _p(out), T, Fh, limit, alpha, _DT[x.dtype], _stream(x)),
+                      "lv_clamped_glu")
+        return out
+    g = x[:, :Fh].float().clamp(max=limit)
+    u = x[:, Fh:].float().clamp(-limit, limit)
+    out.copy_(g * torch.sigmoid(alpha * g) * (u + 1))
+    return out
+
+
+# ------------------------------------------------------------------------------------- delta rule
+def delta_prep(proj, conv_w, conv_state, A_log, dt_bias, step, G, H, D, Dv, taps, off_b, off_a, unit_eps):
+    """Short causal convolution + silu over the q | k | v channels of `proj` [T, ld] (taps from the
+    portion's own rows, then from the carried state of the sequence's slot, zeros before position
+    0), unit-norm q (times D^-1/2) and k per head, beta = sigmoid(b), decay = exp(-exp(A_log) *
+    softplus(a + dt_bias)). Returns f32 (qn [T,G,D], kn [T,G,D], v [T,H,Dv], beta [T,H], decay [T,H])."""
+    T = proj.size(0)
+    dev = proj.device
+    _f32(conv_w, A_log, dt_bias)
+    qn = torch.empty(T, G, D, dtype=torch.float32, device=dev)
+    kn = torch.empty(T, G, D, dtype=torch.float32, device=dev)
+    v = torch.empty(T, H, Dv, dtype=torch.float32, device=dev)
+    beta = torch.empty(T, H, dtype=torch.float32, device=dev)
+    decay = torch.empty(T, H, dtype=torch.float32, device=dev)
+    C = 2 * G * D + H * Dv
+    assert conv_state.is_contiguous() and conv_state.shape[1:] == (taps - 1, C) and conv_state.dtype == proj.dtype
+    if proj.is_cuda:
+        assert proj.stride(1) == 1
+        lib = _mixlib.load()
+        _mixlib.check(lib.lv_delta_prep(_p(proj), proj.stride(0), _p(conv_w), _p(conv_state), _p(A_log), _p(dt_bias),
+                                        _p(step.cu_q), _p(step.ctx_lens), _p(step.slots), _p(step.tok_seq), _p(qn),
+                                        _p(kn), _p(v), _p(beta), _p(decay), T, G, H, D, Dv, taps, off_b, off_a,
+                                        unit_eps, _DT[proj.dtype], _stream(proj)), "lv_delta_prep")
+        return qn, kn, v, beta, decay
+    q0 = 0
+    for b, (n, ctx) in enumerate(zip(step.host_lens_q, step.host_ctx_lens)):
+        rows = proj[q0:q0 + n, :C].float()
+        hist = conv_state[step.host_slots[b]].float() if ctx > 0 else torch.zeros(taps - 1, C)
+        if 0 < ctx < taps - 1:
+            hist = hist.clone()
+            hist[:taps - 1 - ctx] = 0
+        full = torch.cat([hist, rows])
+        y = sum(full[i:i + n] * conv_w[:, i] for i in range(taps))
+        y = F.silu(y)
+        qq = y[:, :G * D].view(n, G, D)
+        kk = y[:, G * D:2 * G * D].view(n, G, D)
+        qn[q0:q0 + n] = qq / torch.sqrt(qq.pow(2).sum(-1, keepdim=True) + unit_eps) * D ** -0.5
+        kn[q0:q0 + n] = kk / torch.sqrt(kk.pow(2).sum(-1, keepdim=True) + unit_eps)
+        v[q0:q0 + n] = y[:, 2 * G * D:].view(n, H, Dv)
+        beta[q0:q0 + n] = torch.sigmoid(proj[q0:q0 + n, off_b:off_b + H].float())
+        decay[q0:q0 + n] = torch.exp(-torch.exp(A_log) * F.softplus(proj[q0:q0 + n, off_a:off_a + H].float() + dt_bias))
+        q0 += n
+    return qn, kn, v, beta, decay
+
+
+def conv_state_update(proj, conv_state, step, C, taps):
+    """conv_state[slot] <- the last taps-1 convolution inputs of every sequence after this step."""
+    if taps <= 1:
+        return
+    if proj.is_cuda:
+        lib = _mixlib.load()
+        _mixlib.check(lib.lv_conv_state_update(_p(proj), proj.stride(0), _p(conv_state), _p(step.cu_q),
+                                               _p(step.ctx_lens), _p(step.slots), len(step.host_lens_q), C, taps,
+                                               _DT[proj.dtype], _stream(proj)), "lv_conv_state_update")
+        return
+    q0 = 0
+    for b, (n, ctx) in enumerate(zip(step.host_lens_q, step.host_ctx_lens)):
+        slot = step.host_slots[b]
+        hist = conv_state[slot].clone() if ctx > 0 else torch.zeros_like(conv_state[slot])
+        if 0 < ctx < taps - 1:
+            hist[:taps - 1 - ctx] = 0
+        full = torch.cat([hist, proj[q0:q0 + n, :C]])
+        conv_state[slot] = full[-(taps - 1):]
+        q0 += n
+
+
+def gated_delta_rule(qn, kn, v, beta, decay, state, step):
+    """Per head and token: S <- decay * S; u = beta * (v - S^T k); S <- S + k u^T; o = S^T q.
+    state f32 [slots, H, D, Dv] (taken as zero for a sequence with no context), updated in place.
+    Returns o f32 [T, H, Dv]."""
+    T, G, D = qn.shape
+    H, Dv = v.shape[1], v.shape[2]
+    _f32(qn, kn, v, beta, decay, state)
+    assert state.shape[1:] == (H, D, Dv)
+    o = torch.empty(T, H, Dv, dtype=torch.float32, device=qn.device)
+    if qn.is_cuda:
+        lib = _mixlib.load()
+        _mixlib.check(lib.lv_gated_delta_rule(_p(qn), _p(kn), _p(v), _p(beta), _p(decay), _p(state), _p(step.cu_q),
+                                              _p(step.ctx_lens), _p(step.slots), _p(o), len(step.host_lens_q), G, H, D,
+                                              Dv, _stream(qn)), "lv_gated_delta_rule")
+        return o
+    rep = H // G
+    q0 = 0
+    for b, (n, ctx) in enumerate(zip(step.host_lens_q, step.host_ctx_lens)):
+        slot = step.host_slots[b]
+        S = state[slot].clone() if ctx > 0 else torch.zeros(H, D, Dv)
+        for t in range(q0, q0 + n):
+            k = kn[t].repeat_interleave(rep, 0)      # [H, D]
+            q = qn[t].repeat_interleave(rep, 0)
+            S = decay[t][:, None, None] * S
+            u = beta[t][:, None] * (v[t] - torch.einsum("hdv,hd->hv", S, k))
+            S = S + k[:, :, None] * u[:, None, :]
+            o[t] = torch.einsum("hdv,hd->hv", S, q)
+        state[slot] = S
+        q0 += n
+    return o
+
+
+def head_norm_gate(o, gate, norm_w, eps, act_dtype):
+    """o f32 [T, H, Dv] -> act [T, H*Dv]: per-head RMS norm over Dv, times norm_w [Dv], times silu(gate)."""
+    T, H, Dv = o.shape
+    _f32(o, norm_w)
+    out = torch.empty(T, H * Dv, dtype=act_dtype, device=o.device)
+    if o.is_cuda:
+        assert gate.stride(1) == 1 and gate.dtype == act_dtype
+        lib = _mixlib.load()
+        _mixlib.check(lib.lv_head_norm_gate(_p(o), _p(gate), gate.stride(0), _p(norm_w), _p(out), T, H, Dv, eps,
+                                            _DT[act_dtype], _stream(o)), "lv_head_norm_gate")
+        return out
+    y = o / torch.sqrt(o.pow(2).mean(-1, keepdim=True) + eps) * norm_w
+    out.copy_((y * F.silu(gate.float()).view(T, H, Dv)).reshape(T, H * Dv))
+    return out
+
+
+# ------------------------------------------------------------------------- windowed pooled attention
+def pooled_slots(page: int, P: int) -> int:
+    """Pooled entries a page can own: blocks whose last token lies in it."""
+    return -(-page // P) if P > 0 else 0
+
+
+def _token_slot(bt_row, j, page):
+    return bt_row[j // page] * page + j % page
+
+
+def _pool_slot(bt_row, blk, page, P, PP):
+    pj = (blk * P + P - 1) // page
+    return bt_row[pj] * PP + blk - (page * pj) // P
+
+
+def qk_fullnorm_store(q, k, v, q_w, k_w, k_cache, v_cache, step, H, G, D, Dv, eps):
+    """RMS norm over the whole q row [H*D] and the whole k row [G*D] (weights q_w, k_w), normed K and
+    V scattered into the paged caches [pages, page, G, D|Dv] at each token's position. Returns normed q."""
+    T = q.size(0)
+    page = k_cache.size(1)
+    _f32(q_w, k_w)
+    q_out = torch.empty(T, H * D, dtype=q.dtype, device=q.device)
+    if q.is_cuda:
+        ld = q.stride(0)
+        assert k.stride(0) == ld and v.stride(0) == ld and q.stride(1) == 1 and k_cache.is_contiguous() and v_cache.is_contiguous()
+        lib = _mixlib.load()
+        _mixlib.check(lib.lv_qk_fullnorm_store(_p(q), _p(k), _p(v), ld, _p(q_w), _p(k_w), _p(q_out), _p(k_cache),
+                                               _p(v_cache), _p(step.cu_q), _p(step.ctx_lens), _p(step.tok_seq),
+                                               _p(step.block_tables), step.block_tables.stride(0), T, H, G, D, Dv, page,
+                                               eps, _DT[q.dtype], _stream(q)), "lv_qk_fullnorm_store")
+        return q_out
+    qf, kf = q.float(), k.float()
+    q_out.copy_(qf / torch.sqrt(qf.pow(2).mean(-1, keepdim=True) + eps) * q_w)
+    kn = (kf / torch.sqrt(kf.pow(2).mean(-1, keepdim=True) + eps) * k_w).to(k_cache.dtype)
+    kc, vc = k_cache.view(-1, G * D), v_cache.view(-1, G * Dv)
+    q0 = 0
+    for b, (n, ctx) in enumerate(zip(step.host_lens_q, step.host_ctx_lens)):
+        bt = step.host_block_tables[b]
+        for r in range(n):
+            s = _token_slot(bt, ctx + r, page)
+            kc[s] = kn[q0 + r]
+            vc[s] = v[q0 + r]
+        q0 += n
+    return q_out
+
+
+def pool_update(k_cache, v_cache, kp, vp, step, G, D, Dv, P):
+    """Means of the P cached keys / values of every block this step completed, stored with the page of
+    the block's last token (kp, vp: [pages, pooled_slots(page, P), G, D|Dv])."""
+    if P <= 0:
+        return
+    page = k_cache.size(1)
+    new_blocks = [(c + n) // P - c // P for n, c in zip(step.host_lens_q, step.host_ctx_lens)]
+    most = max(new_blocks, default=0)
+    if most == 0:
+        return
+    if k_cache.is_cuda:
+        lib = _mixlib.load()
+        _mixlib.check(lib.lv_pool_update(_p(k_cache), _p(v_cache), _p(kp), _p(vp), _p(step.cu_q), _p(step.ctx_lens),
+                                         _p(step.block_tables), step.block_tables.stride(0), len(new_blocks), most, G,
+                                         D, Dv, page, P, _DT[k_cache.dtype], _stream(k_cache)), "lv_pool_update")
+        return
+    PP = pooled_slots(page, P)
+    kc, vc = k_cache.view(-1, G * D), v_cache.view(-1, G * Dv)
+    kpf, vpf = kp.view(-1, G * D), vp.view(-1, G * Dv)
+    for b, (n, ctx) in enumerate(zip(step.host_lens_q, step.host_ctx_lens)):
+        bt = step.host_block_tables[b]
+        for blk in range(ctx // P, (ctx + n) // P):
+            rows = [_token_slot(bt, j, page) for j in range(blk * P, blk * P + P)]
+            dst = _pool_slot(bt, blk, page, P, PP)
+            kpf[dst] = kc[rows].float().mean(0)
+            vpf[dst] = vc[rows].float().mean(0)
+
+
+def window_pool_attention(q, k_cache, v_cache, kp, vp, gate, step, H, G, D, Dv, window, P, scale, has_sink=True):
+    """Query at position i attends to cached positions j with 0 <= i - j < window and to the pooled
+    entry of every block b with b*P + P - 1 <= i - window, one softmax over both, `has_sink` adding 1
+    to its denominator; the result is multiplied by sigmoid(gate) when a gate is given.
+    q [T, H*D] contiguous act; returns act [T, H*Dv]."""
+    T = q.size(0)
+    page = k_cache.size(1)
+    out = torch.empty(T, H * Dv, dtype=q.dtype, device=q.device)
+    if q.is_cuda:
+        assert q.is_contiguous() and (gate is None or gate.stride(1) == 1)
+        lib = _mixlib.load()
+        _mixlib.check(lib.lv_window_pool_attn(_p(q), _p(k_cache), _p(v_cache), _p(kp), _p(vp), _p(gate),
+                                              gate.stride(0) if gate is not None else 0, _p(out), _p(step.cu_q),
+                                              _p(step.ctx_lens), _p(step.tok_seq), _p(step.block_tables),
+                                              step.block_tables.stride(0), T, H, G, D, Dv, page, window, P, scale,
+                                              int(has_sink), _DT[q.dtype], _stream(q)), "lv_window_pool_attn")
+        return out
+    PP = pooled_slots(page, P)
+    rep = H // G
+    kc, vc = k_cache.view(-1, G, D), v_cache.view(-1, G, Dv)
+    q0 = 0
+    for b, (n, ctx) in enumerate(zip(step.host_lens_q, step.host_ctx_lens)):
+        bt = step.host_block_tables[b]
+        for r in range(n):
+            i = ctx + r
+            nb = max(0, (i - window + 1) // P) if P > 0 else 0
+            rows = [_token_slot(bt, j, page) for j in range(max(0, i - window + 1), i + 1)]
+            K, V = kc[rows].float(), vc[rows].float()
+            if nb:
+                prow = [_pool_slot(bt, blk, page, P, PP) for blk in range(nb)]
+                K = torch.cat([kp.view(-1, G, D)[prow].float(), K])
+                V = torch.cat([vp.view(-1, G, Dv)[prow].float(), V])
+            qi = q[q0 + r].float().view(G, rep, D)
+            s = torch.einsum("grd,ngd->grn", qi, K) * scale
+            m = s.max(-1, keepdim=True).values.clamp(min=0)
+            e = torch.exp(s - m)
+            w = e / (e.sum(-1, keepdim=True) + (torch.exp(-m) if has_sink else 0))
+            o = torch.einsum("grn,ngv->grv", w, V).reshape(H * Dv)
+            if gate is not None:
+                o = o * torch.sigmoid(gate[q0 + r].float())
+            out[q0 + r] = o
+        q0 += n
+    return out

@@ -16,8 +16,20 @@ def default_weight_loader(param: nn.Parameter, loaded_weight: torch.Tensor):
     param.data.copy_(loaded_weight)
 
 
+def checkpoint_tensors(path: str):
+    """(name, tensor) pairs of every *.safetensors file of a directory, read one tensor at a time."""
+    from safetensors import safe_open
+    for file in sorted(glob(os.path.join(path, "*.safetensors"))):
+        with safe_open(file, "pt", "cpu") as f:
+            for name in f.keys():
+                yield name, f.get_tensor(name)
+
+
 def load_model(model: nn.Module, path: str) -> None:
     from safetensors import safe_open
+    if hasattr(model, "load_weights"):       # models with their own checkpoint naming place the tensors themselves
+        model.load_weights(checkpoint_tensors(path))
+        return
     packed = getattr(model, "packed_modules_mapping", {})
     for file in sorted(glob(os.path.join(path, "*.safetensors"))):
         with safe_open(file, "pt", "cpu") as f:
@@ -143,6 +155,9 @@ def lagcopy_checkpoint(hf_config, seed: int = 0):
 def load_random(model: nn.Module, hf_config, seed: int = 0, std: float = 0.02, kind: str = "normal") -> None:
     """Fill `model` (any TP shard of it) from random_checkpoint (kind "normal") or lagcopy_checkpoint
     (kind "lagcopy") through the weight loaders."""
+    if hasattr(model, "load_weights"):
+        model.load_weights(model.random_weights(seed))
+        return
     packed = getattr(model, "packed_modules_mapping", {})
     source = lagcopy_checkpoint(hf_config, seed) if kind == "lagcopy" else random_checkpoint(hf_config, seed, std)
     for name, tensor in source:
