@@ -1,0 +1,51 @@
+"""Kagalorn on the GPU: the HIP kernels of liblvmix.so, alone and through the engine, against the oracle."""
+import pytest
+
+from tests import _kagalorn as K
+from tests import _kagalorn_cases as C
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+DTYPES = ["float32", "bfloat16"]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_mechanisms(gpu, dtype):
+    C.case_hyper_connection_and_norm(DEV, dtype)
+    C.case_clamped_glu(DEV, dtype)
+    C.case_head_norm_gate(DEV, dtype)
+    C.case_qk_norm_store(DEV, dtype)
+    C.case_sink_and_gate(DEV, dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_delta_rule_portions(gpu, dtype):
+    C.case_delta_rule_portions(DEV, dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_window_pool_beacons(gpu, dtype):
+    C.case_window_pool_beacons(DEV, dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_engine_schedules(gpu, tmp_path, dtype):
+    C.case_engine_schedules(DEV, dtype, tmp_path)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_engine_odd_sizes(gpu, tmp_path, dtype):
+    C.case_engine_schedules(DEV, dtype, tmp_path, cfg=K.CFG_ODD, seed=9)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_engine_reuse_of_pages_and_slots(gpu, tmp_path, dtype):
+    C.case_engine_reuse(DEV, dtype, tmp_path)
+
+
+def test_engine_long_decode(gpu, tmp_path):
+    C.case_engine_long_decode(DEV, "float32", tmp_path)
+
+
+def test_generate_greedy(gpu, tmp_path):
+    C.case_generate(DEV, tmp_path)
