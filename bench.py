@@ -562,6 +562,180 @@ def e2e_leg(n, port, mode, limit_s, tuned_gemms=False):
     return {"mode": mode, "error": f"exit code {proc.returncode}: {err.strip()[-300:]}"}
 
 
+# ------------------------------------------------------------------------------------------------
+# --mixers: the Kagalorn design (delta-rule and windowed pooled attention layers on hyper-connected
+# streams) beside Qwen3 at equal width, depth and head counts, both with random weights, through the
+# engine (LLM.generate: prefill and decode tok/s), and the design's kernels one by one at the same
+# layer shapes beside the Qwen3 kernel that does the like job, each against its own roofline
+# (HBM bytes at 8 TB/s for the memory-bound ones, dense bf16 MFMA rate for prompt attention).
+MIXER_SIZES = {
+    "2k": dict(width=2048, layers=8, heads=16, kv_heads=4, dim=128, ff=6144, window=1024, pool=64, vocab=32000),
+    "4k": dict(width=4096, layers=4, heads=32, kv_heads=8, dim=128, ff=12288, window=2048, pool=128, vocab=32000),
+}
+HBM_BPS, MFMA_FLOPS = 8.0e12, 2.5e15
+
+
+def _kagalorn_config(z):
+    from light_vllm_amd.models.kagalorn import KagalornConfig
+    att = {"heads": z["heads"], "kv_heads": z["kv_heads"], "dim": z["dim"], "vdim": z["dim"], "scale": z["dim"] ** -0.5,
+           "mask": {"size": z["window"], "pool": z["pool"]}}
+    dlt = {"heads": z["heads"], "kv_heads": z["kv_heads"], "dim": z["dim"], "vdim": z["dim"], "conv": 4}
+    mlp = {"kind": "dense", "ff": z["ff"], "limit": 7.0}
+    layers = [{"type": "delta" if i % 2 == 0 else "attention", "mixer": dlt if i % 2 == 0 else att, "mlp": mlp}
+              for i in range(z["layers"])]
+    return KagalornConfig.from_dict({"vocab": z["vocab"], "width": z["width"], "streams": 4,
+                                     "norm": {"eps": 1e-6, "groups": 4}, "layers": layers})
+
+
+def _qwen3_config(z):
+    from types import SimpleNamespace
+    return SimpleNamespace(vocab_size=z["vocab"], head_dim=z["dim"], hidden_act="silu", max_position_embeddings=40960,
+                           rms_norm_eps=1e-6, rope_theta=1000000, rope_scaling=None, attention_bias=False,
+                           torch_dtype=torch.bfloat16, hidden_size=z["width"], intermediate_size=z["ff"],
+                           num_hidden_layers=z["layers"], num_attention_heads=z["heads"],
+                           num_key_value_heads=z["kv_heads"], tie_word_embeddings=False)
+
+
+def _engine_rates(hf_config, batch, prompt_len, new_tokens, **kw):
+    from light_vllm_amd.llm import LLM
+    from light_vllm_amd.sampling_params import SamplingParams
+    g = torch.Generator().manual_seed(0)
+    prompts = [torch.randint(0, hf_config.vocab_size, (prompt_len,), generator=g).tolist() for _ in range(batch)]
+    llm = LLM(None, hf_config=hf_config, max_num_seqs=batch, max_model_len=4096, max_num_batched_tokens=16384,
+              random_seed=0, random_on_device=True, **kw)
+    llm.generate(prompts[:2], SamplingParams(temperature=0.0, max_tokens=2, ignore_eos=True))      # warm the libraries
+    llm.generate(prompts, SamplingParams(temperature=0.0, max_tokens=new_tokens, ignore_eos=True))
+    st = dict(llm.last_stats)
+    llm.exit()
+    del llm
+    torch.cuda.empty_cache()
+    return {"prefill_tok_s": round(st["avg_prefill_tok_s"], 1), "decode_tok_s": round(st["avg_decode_tok_s"], 1)}
+
+
+def _mixer_kernel_table(z, dev, batch, prompt_len):
+    """Each kernel of the design alone, at one layer's shapes: a prompt step (batch x prompt_len new tokens)
+    and a decode step (batch single tokens behind prompt_len tokens), with the Qwen3 kernel of the like job."""
+    from light_vllm_amd import mix_ops, ops
+    from light_vllm_amd.utils.context import RaggedStep
+    bf = torch.bfloat16
+    W, H, G, D, F_, S = z["width"], z["heads"], z["kv_heads"], z["dim"], z["ff"], 4
+    window, P, page = z["window"], z["pool"], 256
+    rows = []
+
+    def step_of(lens_q, ctx):
+        B = len(lens_q)
+        cu = [0]
+        tok = []
+        for b, n_ in enumerate(lens_q):
+            cu.append(cu[-1] + n_)
+            tok += [b] * n_
+        per = -(-(max(ctx) + max(lens_q)) // page)
+        tables = [[b * per + j for j in range(per)] for b in range(B)]
+        i32 = dict(dtype=torch.int32, device=dev)
+        return RaggedStep(torch.tensor(cu, **i32), torch.tensor(ctx, **i32), torch.arange(B, **i32),
+                          torch.tensor(tok, **i32), torch.tensor(tables, **i32), lens_q, ctx, list(range(B)), tables), B * per
+
+    def add(name, phase, fn, nbytes=0, flops=0, like=None):
+        us = _event_time(fn, 20, 3) * 1e6
+        rec = {"kernel": name, "phase": phase, "us": round(us, 1)}
+        if nbytes:
+            rec["GBs"] = round(nbytes / us / 1e3, 1)
+            rec["of_hbm_roofline"] = round(nbytes / us / 1e3 / (HBM_BPS / 1e9), 3)
+        if flops:
+            rec["TFLOPs"] = round(flops / us / 1e6, 2)
+            rec["of_mfma_roofline"] = round(flops / us / 1e6 / (MFMA_FLOPS / 1e12), 4)
+        if like:
+            rec["like"] = like
+        rows.append(rec)
+
+    for phase, lens_q, ctx in (("prompt", [prompt_len] * batch, [0] * batch), ("decode", [1] * batch, [prompt_len] * batch)):
+        step, pages = step_of(lens_q, ctx)
+        T = sum(lens_q)
+        x = torch.randn(T, S, W, device=dev)
+        y = torch.randn(T, W, device=dev, dtype=bf)
+        mixm, vec, nw = torch.eye(S, device=dev), torch.ones(S, device=dev), torch.ones(W, device=dev)
+        add("hc_update_norm", phase, lambda: mix_ops.hc_update_norm(x, y, mixm, vec, vec, nw, 4, 1e-6, bf),
+            nbytes=T * W * (8 * S + 4))
+        res = torch.randn(T, W, device=dev, dtype=bf)
+        nwb = torch.ones(W, device=dev, dtype=bf)
+        add("qwen3 add_rms_norm", phase, lambda: ops.add_rms_norm(y, res, nwb, 1e-6), nbytes=T * W * 8, like="hc_update_norm")
+        gu = torch.randn(T, 2 * F_, device=dev, dtype=bf)
+        add("clamped_glu", phase, lambda: mix_ops.clamped_glu(gu, 7.0, 1.702), nbytes=T * F_ * 6)
+        add("qwen3 silu_and_mul", phase, lambda: ops.silu_and_mul(gu), nbytes=T * F_ * 6, like="clamped_glu")
+        # delta rule
+        C = 2 * G * D + H * D
+        ld = C + H * D + 2 * H
+        proj = torch.randn(T, ld, device=dev, dtype=bf)
+        conv_w = torch.randn(C, 4, device=dev) * 0.5
+        conv_state = torch.zeros(batch, 3, C, device=dev, dtype=bf)
+        A_log, dt_bias = torch.zeros(H, device=dev), torch.zeros(H, device=dev)
+        state = torch.zeros(batch, H, D, D, device=dev)
+        add("delta_prep", phase, lambda: mix_ops.delta_prep(proj, conv_w, conv_state, A_log, dt_bias, step, G, H, D, D, 4,
+                                                            C + H * D, C + H * D + H, 1e-6),
+            nbytes=T * (C * 2 + C * 4 + 8 * H))
+        qn, kn, v, beta, dec = mix_ops.delta_prep(proj, conv_w, conv_state, A_log, dt_bias, step, G, H, D, D, 4,
+                                                  C + H * D, C + H * D + H, 1e-6)
+        st_bytes = batch * H * D * D * 4 * 2
+        add("gated_delta_rule", phase, lambda: mix_ops.gated_delta_rule(qn, kn, v, beta, dec, state, step),
+            nbytes=st_bytes + T * (2 * G * D + 2 * H * D) * 4, flops=T * H * D * D * 2 * 3)
+        o32 = torch.randn(T, H, D, device=dev)
+        add("head_norm_gate", phase, lambda: mix_ops.head_norm_gate(o32, proj[:, C:C + H * D], nw[:D].contiguous(), 1e-6, bf),
+            nbytes=T * H * D * 8)
+        # windowed pooled attention
+        qkv = torch.randn(T, (H + 2 * G) * D + H * D, device=dev, dtype=bf)
+        kc = torch.zeros(pages, page, G, D, device=dev, dtype=bf)
+        vc = torch.zeros(pages, page, G, D, device=dev, dtype=bf)
+        pp = mix_ops.pooled_slots(page, P)
+        kp, vp = torch.zeros(pages, pp, G, D, device=dev, dtype=bf), torch.zeros(pages, pp, G, D, device=dev, dtype=bf)
+        qw, kw_ = torch.ones(H * D, device=dev), torch.ones(G * D, device=dev)
+        a_, b_, c_ = H * D, (H + G) * D, (H + 2 * G) * D
+        add("qk_fullnorm_store", phase, lambda: mix_ops.qk_fullnorm_store(qkv[:, :a_], qkv[:, a_:b_], qkv[:, b_:c_], qw, kw_, kc, vc,
+                                                                         step, H, G, D, D, 1e-6),
+            nbytes=T * (H + 2 * G) * D * 4)
+        qn_ = mix_ops.qk_fullnorm_store(qkv[:, :a_], qkv[:, a_:b_], qkv[:, b_:c_], qw, kw_, kc, vc, step, H, G, D, D, 1e-6)
+        add("pool_update", phase, lambda: mix_ops.pool_update(kc, vc, kp, vp, step, G, D, D, P))
+        keys = sum(min(i + 1, window) + max(0, (i - window + 1) // P) for n_, c0 in zip(lens_q, ctx) for i in range(c0, c0 + n_))
+        if phase == "prompt":
+            add("window_pool_attn", phase, lambda: mix_ops.window_pool_attention(qn_, kc, vc, kp, vp, qkv[:, c_:], step, H, G, D, D,
+                                                                               window, P, D ** -0.5, True),
+                flops=keys * H * D * 4)
+        else:
+            add("window_pool_attn", phase, lambda: mix_ops.window_pool_attention(qn_, kc, vc, kp, vp, qkv[:, c_:], step, H, G, D, D,
+                                                                               window, P, D ** -0.5, True),
+                nbytes=keys * G * D * 4)
+        # the Qwen3 attention at the same shapes: full causal prompt attention / full-context decode
+        q3 = torch.randn(T, H, D, device=dev, dtype=bf)
+        k3 = torch.randn(T, G, D, device=dev, dtype=bf)
+        if phase == "prompt":
+            cu3 = torch.tensor([i * prompt_len for i in range(batch + 1)], dtype=torch.int32, device=dev)
+            add("qwen3 prefill_attn", phase, lambda: ops.prefill_attention(q3, k3, k3, cu3, cu3, prompt_len, prompt_len, D ** -0.5),
+                flops=batch * prompt_len * (prompt_len + 1) // 2 * H * D * 4, like="window_pool_attn")
+        else:
+            cl = torch.full((batch,), prompt_len + 1, dtype=torch.int32, device=dev)
+            bt3 = step.block_tables
+            add("qwen3 decode_attn", phase, lambda: ops.decode_attention(q3, kc, vc, cl, bt3, D ** -0.5),
+                nbytes=batch * (prompt_len + 1) * G * D * 4, like="window_pool_attn")
+    return rows
+
+
+def mixers_leg(sizes, batch, prompt_len, new_tokens):
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    out = {"metric": "mixers: Kagalorn beside Qwen3 at equal size", "dtype": "bf16", "data": "synthetic, random weights",
+           "batch": batch, "prompt_len": prompt_len, "new_tokens": new_tokens, "sizes": []}
+    for name in sizes:
+        z = MIXER_SIZES[name]
+        rec = {"size": name, **z}
+        rec["kagalorn"] = _engine_rates(_kagalorn_config(z), batch, prompt_len, new_tokens, kvcache_block_size=256,
+                                        max_cache_tokens=batch * 256 * (-(-(prompt_len + new_tokens) // 256)))
+        blocks = batch * (-(-(prompt_len + new_tokens) // 256)) + 8
+        rec["qwen3_eager"] = _engine_rates(_qwen3_config(z), batch, prompt_len, new_tokens, num_kvcache_blocks=blocks,
+                                           enforce_eager=True)
+        rec["kernels"] = _mixer_kernel_table(z, dev, batch, prompt_len)
+        out["sizes"].append(rec)
+    print(json.dumps(out), flush=True)
+
+
 def tp_step_setup(ops, dev, n, rank, cfg, layers, batch):
     """The config-4 step on this rank: workload + the activation the per-layer all-reduce sums."""
     w = DecodeWorkload(ops, dev, layers, cfg["hq"] // n, cfg["hkv"] // n, batch, cfg["ctx"], seed=4321 + rank)
@@ -608,7 +782,14 @@ def main():
     ap.add_argument("--rehearse", action="store_true",
                     help="N > 1 on ONE GPU: every rank on cuda:0, gloo group, 4 layers, batch 8 "
                          "(proves launcher, rendezvous, graph and JSON path; not a measurement)")
+    ap.add_argument("--mixers", default="", help="comma list of sizes (2k, 4k): instead of the contract workload, "
+                    "run the Kagalorn design beside Qwen3 at equal size and time its kernels one by one")
+    ap.add_argument("--mixers-batch", type=int, default=16)
+    ap.add_argument("--mixers-prompt", type=int, default=1024)
+    ap.add_argument("--mixers-new", type=int, default=17)
     args = ap.parse_args()
+    if args.mixers:
+        return mixers_leg([x for x in args.mixers.split(",") if x], args.mixers_batch, args.mixers_prompt, args.mixers_new)
 
     aux = set() if args.no_aux else {a for a in args.aux.split(",") if a}
     world = int(os.environ.get("WORLD_SIZE", "1"))

@@ -373,7 +373,7 @@ int lv_delta_prep(const void* proj, int64_t ld, const void* conv_w, const void* 
                   const int32_t* tok_seq, void* qn, void* kn, void* v, void* beta, void* decay, int64_t T, int G,
                   int H, int D, int Dv, int taps, int off_b, int off_a, float unit_eps, int dtype, void* stream) {
   if (T == 0) return 0;
-  if (!proj || !conv_w || !conv_state || !A_log || !dt_bias || !cu_q || !ctx_lens || !slots || !tok_seq || !qn ||
+  if (!proj || !conv_w || (!conv_state && taps > 1) || !A_log || !dt_bias || !cu_q || !ctx_lens || !slots || !tok_seq || !qn ||
       !kn || !v || !beta || !decay)
     return fail(-1, "lv_delta_prep: null pointer");
   if (G <= 0 || H <= 0 || H % G != 0 || D <= 0 || Dv <= 0 || taps < 1) return fail(-1, "lv_delta_prep: bad sizes");

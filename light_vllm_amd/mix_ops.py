@@ -18,6 +18,9 @@ import torch.nn.functional as F
 from . import _mixlib
 
 _DT = {torch.bfloat16: 0, torch.float32: 1}
+# windowed pooled attention: "auto" takes the matrix-core kernel where it applies (bf16, head sizes that
+# are multiples of 16 up to 256) and the vector kernel elsewhere (f32, other head sizes); "valu" forces the latter
+WINDOW_ATTN_KERNEL = "auto"
 
 
 def _stream(t: torch.Tensor) -> int:
@@ -275,6 +278,15 @@ def window_pool_attention(q, k_cache, v_cache, kp, vp, gate, step, H, G, D, Dv, 
     if q.is_cuda:
         assert q.is_contiguous() and (gate is None or gate.stride(1) == 1)
         lib = _mixlib.load()
+        if (WINDOW_ATTN_KERNEL == "auto" and q.dtype == torch.bfloat16 and D % 16 == 0 and Dv % 16 == 0
+                and D <= 256 and Dv <= 256):
+            _mixlib.check(lib.lv_window_pool_attn_mfma(_p(q), _p(k_cache), _p(v_cache), _p(kp), _p(vp), _p(gate),
+                                                       gate.stride(0) if gate is not None else 0, _p(out), _p(step.cu_q),
+                                                       _p(step.ctx_lens), _p(step.block_tables),
+                                                       step.block_tables.stride(0), len(step.host_lens_q),
+                                                       max(step.host_lens_q), H, G, D, Dv, page, window, P, scale,
+                                                       int(has_sink), _stream(q)), "lv_window_pool_attn_mfma")
+            return out
         _mixlib.check(lib.lv_window_pool_attn(_p(q), _p(k_cache), _p(v_cache), _p(kp), _p(vp), _p(gate),
                                               gate.stride(0) if gate is not None else 0, _p(out), _p(step.cu_q),
                                               _p(step.ctx_lens), _p(step.tok_seq), _p(step.block_tables),

@@ -242,6 +242,27 @@ class KagalornForCausalLM(nn.Module):
         if missing:
             raise KeyError(f"checkpoint lacks {missing[:8]}{' ...' if len(missing) > 8 else ''}")
 
+    @torch.no_grad()
+    def init_random_on_device(self, seed: int = 0) -> None:
+        """Fast random fill on the parameters' own device (benchmarks: values differ between devices)."""
+        S = self.config.streams
+        gens = {}
+        for name, (param, where, _) in self.weight_targets().items():
+            if where is not None and not (isinstance(where, int) and where == 0) and not (isinstance(where, tuple) and where[1] == 0):
+                continue                    # merged tensors are filled once, through their first part
+            g = gens.get(param.device)
+            if g is None:
+                g = gens[param.device] = torch.Generator(device=param.device).manual_seed(seed)
+            leaf = name.rsplit(".", 1)[-1]
+            if "norm" in leaf:
+                param.fill_(1.0)
+            elif ".hc" in name:
+                param.copy_(torch.eye(S) if leaf == "mix" else torch.full((S,), 1.0 / S if leaf == "in" else 1.0))
+            elif leaf in ("conv", "A_log", "dt_bias"):
+                param.normal_(0.0, 0.5, generator=g)
+            else:
+                param.normal_(0.0, param.shape[-1] ** -0.5, generator=g)
+
     def random_weights(self, seed: int = 0):
         """(name, tensor) pairs of a seeded random checkpoint of this configuration, for runs without
         weights on disk. Scales keep activations of order one through any depth."""

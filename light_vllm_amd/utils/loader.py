@@ -174,6 +174,9 @@ def load_random(model: nn.Module, hf_config, seed: int = 0, std: float = 0.02, k
 def load_random_on_device(model: nn.Module, seed: int = 0, std: float = 0.02) -> None:
     """Fast random fill on the parameters' own device (benchmarks only: values differ between
     devices and TP layouts, unlike load_random). Norm weights are set to one."""
+    if hasattr(model, "init_random_on_device"):
+        model.init_random_on_device(seed)
+        return
     dev_gens = {}
     for name, param in model.named_parameters():
         if name.endswith("norm.weight") or "layernorm" in name:

@@ -41,6 +41,19 @@ CFG_ODD = {
 }
 
 
+# head sizes in multiples of 16 (in bf16 the attention layers then run on the matrix cores), five query heads a kv head
+CFG_WIDE = {
+    "architecture": "Kagalorn", "vocab": 83, "width": 64, "streams": 2, "norm": {"eps": 1e-6, "groups": 2},
+    "layers": [
+        {"type": "attention", "mixer": {"heads": 5, "kv_heads": 1, "dim": 32, "vdim": 16, "scale": 0.18,
+                                        "mask": {"size": 20, "pool": 6}}, "mlp": {"kind": "dense", "ff": 96, "limit": 3.0}},
+        {"type": "delta", "mixer": {"heads": 2, "kv_heads": 1, "dim": 16, "vdim": 32, "conv": 4}, "mlp": None},
+        {"type": "attention", "mixer": {"heads": 4, "kv_heads": 2, "dim": 16, "vdim": 48, "scale": 0.25,
+                                        "mask": {"size": 17, "pool": 3}}, "mlp": {"kind": "dense", "ff": 96, "limit": 3.0}},
+    ],
+}
+
+
 def write_model(path, cfg: dict, weights: dict) -> str:
     from safetensors.torch import save_file
     os.makedirs(path, exist_ok=True)
@@ -92,7 +105,16 @@ def rel_err(got, want):
 # f32 runs are the sharp comparison. A model this narrow averages little rounding away, so in bf16 single
 # positions are a tenth off the oracle; those runs guard the bf16 kernels against gross faults, the
 # beacon cases (single kernels, scores that stand out) against fine ones.
-TOL = {"float32": 3e-4, "bfloat16": 0.3}
+TOL = {"float32": 3e-4, "bfloat16": 0.5}
+TOL_MEDIAN = {"float32": 1e-4, "bfloat16": 0.12}
+
+
+def assert_close(got, want, dtype, what):
+    d = got.double() - want.double()
+    d = d - d.mean(-1, keepdim=True)
+    w = want.double() - want.double().mean(-1, keepdim=True)
+    e = d.pow(2).mean(-1).sqrt() / w.pow(2).mean().sqrt()
+    assert e.max().item() <= TOL[dtype] and e.median().item() <= TOL_MEDIAN[dtype], (what, e.max().item(), e.median().item())
 
 
 def make_step(lens_q, ctx_lens, slots, tables, device):

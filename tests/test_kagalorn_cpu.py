@@ -34,6 +34,10 @@ def test_engine_odd_sizes(tmp_path):
     C.case_engine_schedules(DEV, "float32", tmp_path, cfg=K.CFG_ODD, seed=9)
 
 
+def test_engine_wide_heads(tmp_path):
+    C.case_engine_schedules(DEV, "float32", tmp_path, cfg=K.CFG_WIDE, seed=11)
+
+
 def test_engine_reuse_of_pages_and_slots(tmp_path):
     C.case_engine_reuse(DEV, "float32", tmp_path)
 

@@ -39,6 +39,22 @@ def test_engine_odd_sizes(gpu, tmp_path, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+def test_engine_wide_heads(gpu, tmp_path, dtype):
+    C.case_engine_schedules(DEV, dtype, tmp_path, cfg=K.CFG_WIDE, seed=11)
+
+
+def test_matrix_core_attention_agrees_with_the_vector_kernel(gpu, tmp_path):
+    """The same bf16 schedules with the vector kernel forced: both kernels serve one model alike."""
+    from light_vllm_amd import mix_ops
+    old, mix_ops.WINDOW_ATTN_KERNEL = mix_ops.WINDOW_ATTN_KERNEL, "valu"
+    try:
+        C.case_engine_schedules(DEV, "bfloat16", tmp_path, cfg=K.CFG_WIDE, seed=11)
+        C.case_window_pool_beacons(DEV, "bfloat16")
+    finally:
+        mix_ops.WINDOW_ATTN_KERNEL = old
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_engine_reuse_of_pages_and_slots(gpu, tmp_path, dtype):
     C.case_engine_reuse(DEV, dtype, tmp_path)
 
