@@ -132,6 +132,37 @@ __global__ __launch_bounds__(256) void clamped_glu_kernel(const T* __restrict__ 
   stf(out + idx, g * sigmoidf_(alpha * g) * (u + 1.0f));
 }
 
+// bf16 rows whose halves start on 16-byte boundaries: eight elements per thread, 16-byte loads and stores.
+__global__ __launch_bounds__(256) void clamped_glu_bf16x8_kernel(const uint16_t* __restrict__ in, int64_t ld_in,
+                                                                 uint16_t* __restrict__ out, int64_t Tn, int F8,
+                                                                 float limit, float alpha) {
+  const int64_t idx = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (idx >= Tn * F8) return;
+  const int64_t t = idx / F8;
+  const int f = static_cast<int>(idx - t * F8) * 8;
+  const uint4 gv = *reinterpret_cast<const uint4*>(in + t * ld_in + f);
+  const uint4 uv = *reinterpret_cast<const uint4*>(in + t * ld_in + static_cast<int64_t>(F8) * 8 + f);
+  const uint32_t gw[4] = {gv.x, gv.y, gv.z, gv.w}, uw[4] = {uv.x, uv.y, uv.z, uv.w};
+  uint32_t ow[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    float r[2];
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+      const float gx = __builtin_bit_cast(float, half ? (gw[i] & 0xffff0000u) : (gw[i] << 16));
+      const float ux = __builtin_bit_cast(float, half ? (uw[i] & 0xffff0000u) : (uw[i] << 16));
+      const float g = fminf(gx, limit);
+      const float u = fminf(fmaxf(ux, -limit), limit);
+      r[half] = g * sigmoidf_(alpha * g) * (u + 1.0f);
+    }
+    bf16_t lo, hi;
+    stf(&lo, r[0]);
+    stf(&hi, r[1]);
+    ow[i] = static_cast<uint32_t>(lo.bits) | (static_cast<uint32_t>(hi.bits) << 16);
+  }
+  *reinterpret_cast<uint4*>(out + idx * 8) = uint4{ow[0], ow[1], ow[2], ow[3]};
+}
+
 // ------------------------------------------------------------------------------------------------
 struct DeltaPrepParams {
   const void* proj;
@@ -236,10 +267,22 @@ struct DeltaRuleParams {
 };
 
 // DR = rows of the state each of the four waves owns (4 * DR >= D; rows beyond D stay zero).
+// Tokens are taken in chunks of kDeltaChunk: the chunk's unit keys and queries, values, write strengths and
+// decays are staged in LDS by all threads at once (one round of global latency per chunk instead of one
+// per token), then each token costs LDS reads, 2 * DR multiply-adds per lane and one barrier.
+constexpr int kDeltaChunk = 16;
+
 template <int DR>
 __global__ __launch_bounds__(256) void gated_delta_rule_kernel(DeltaRuleParams p) {
-  __shared__ float part_k[2][4][kWave];
-  __shared__ float part_o[2][4][kWave];
+  extern __shared__ __attribute__((aligned(16))) float dl[];
+  constexpr int DP = 4 * DR;                       // padded key size
+  float* k_lds = dl;                               // [chunk][DP]
+  float* q_lds = k_lds + kDeltaChunk * DP;         // [chunk][DP]
+  float* v_lds = q_lds + kDeltaChunk * DP;         // [chunk][64]
+  float* bd_lds = v_lds + kDeltaChunk * kWave;     // [chunk][2]: beta, decay
+  float* part_k = bd_lds + kDeltaChunk * 2;        // [2][4][64]
+  float* part_o = part_k + 2 * 4 * kWave;          // [2][4][64]
+  float* o_lds = part_o + 2 * 4 * kWave;           // [chunk][64]: read-outs leave for memory once per chunk
   const int lane = threadIdx.x % kWave, rp = threadIdx.x / kWave;
   const int col = blockIdx.x * kWave + lane;
   const int h = blockIdx.y, b = blockIdx.z;
@@ -255,53 +298,82 @@ __global__ __launch_bounds__(256) void gated_delta_rule_kernel(DeltaRuleParams p
   for (int r = 0; r < DR; ++r)
     s[r] = (carry && live && row0 + r < p.D) ? sbase[static_cast<int64_t>(row0 + r) * p.Dv + col] : 0.0f;
 
-  for (int i = 0; i < n; ++i) {
-    const int64_t t = q0 + i;
-    const int buf = i & 1;
-    const float* kt = p.kn + (t * p.G + g) * p.D;
-    const float* qt = p.qn + (t * p.G + g) * p.D;
-    float kr[DR], qr[DR];
-#pragma unroll
-    for (int r = 0; r < DR; ++r) {
-      const bool in = row0 + r < p.D;
-      kr[r] = in ? kt[row0 + r] : 0.0f;
-      qr[r] = in ? qt[row0 + r] : 0.0f;
+  for (int c0 = 0; c0 < n; c0 += kDeltaChunk) {
+    const int cn = min(kDeltaChunk, n - c0);
+    __syncthreads();                               // the previous chunk is consumed (its last read-out included)
+    for (int x = threadIdx.x; x < cn * DP; x += blockDim.x) {
+      const int tok = x / DP, d = x - tok * DP;
+      const int64_t t = q0 + c0 + tok;
+      const bool in = d < p.D;
+      k_lds[x] = in ? p.kn[(t * p.G + g) * p.D + d] : 0.0f;
+      q_lds[x] = in ? p.qn[(t * p.G + g) * p.D + d] : 0.0f;
     }
-    const float beta = p.beta[t * p.H + h];
-    const float dec = p.decay[t * p.H + h];
-    const float vv = live ? p.v[(t * p.H + h) * p.Dv + col] : 0.0f;
-    float pk = 0.0f;
-#pragma unroll
-    for (int r = 0; r < DR; ++r) pk += s[r] * kr[r];
-    part_k[buf][rp][lane] = pk;
+    for (int x = threadIdx.x; x < cn * kWave; x += blockDim.x) {
+      const int tok = x / kWave, cc = blockIdx.x * kWave + (x % kWave);
+      const int64_t t = q0 + c0 + tok;
+      v_lds[x] = cc < p.Dv ? p.v[(t * p.H + h) * p.Dv + cc] : 0.0f;
+    }
+    if (threadIdx.x < cn) {
+      const int64_t t = q0 + c0 + threadIdx.x;
+      bd_lds[threadIdx.x * 2] = p.beta[t * p.H + h];
+      bd_lds[threadIdx.x * 2 + 1] = p.decay[t * p.H + h];
+    }
     __syncthreads();
-    // the previous token's read-out partials are complete behind this barrier as well
-    if (i > 0 && rp == ((i - 1) & 3) && live) {
-      const int pb = buf ^ 1;
-      p.o[((t - 1) * p.H + h) * p.Dv + col] = part_o[pb][0][lane] + part_o[pb][1][lane] + part_o[pb][2][lane] + part_o[pb][3][lane];
-    }
-    const float ks = part_k[buf][0][lane] + part_k[buf][1][lane] + part_k[buf][2][lane] + part_k[buf][3][lane];
-    const float u = beta * (vv - dec * ks);         // the state is decayed before it is read
-    float po = 0.0f;
+    for (int i = 0; i < cn; ++i) {
+      const int buf = i & 1;
+      float kr[DR], qr[DR];
 #pragma unroll
-    for (int r = 0; r < DR; ++r) {
-      s[r] = dec * s[r] + kr[r] * u;
-      po += s[r] * qr[r];
+      for (int r = 0; r < DR; r += 4) {
+        const float4 k4 = *reinterpret_cast<const float4*>(k_lds + i * DP + row0 + r);
+        const float4 q4 = *reinterpret_cast<const float4*>(q_lds + i * DP + row0 + r);
+        kr[r] = k4.x; kr[r + 1] = k4.y; kr[r + 2] = k4.z; kr[r + 3] = k4.w;
+        qr[r] = q4.x; qr[r + 1] = q4.y; qr[r + 2] = q4.z; qr[r + 3] = q4.w;
+      }
+      const float beta = bd_lds[i * 2], dec = bd_lds[i * 2 + 1];
+      const float vv = v_lds[i * kWave + lane];
+      float pk4[4] = {0.0f, 0.0f, 0.0f, 0.0f};     // four chains: the sums are latency-bound otherwise
+#pragma unroll
+      for (int r = 0; r < DR; ++r) pk4[r & 3] += s[r] * kr[r];
+      part_k[(buf * 4 + rp) * kWave + lane] = (pk4[0] + pk4[1]) + (pk4[2] + pk4[3]);
+      __syncthreads();
+      // the previous token's read-out partials are complete behind this barrier as well
+      if (i > 0 && rp == ((i - 1) & 3)) {
+        const float* po_ = part_o + (buf ^ 1) * 4 * kWave + lane;
+        o_lds[(i - 1) * kWave + lane] = po_[0] + po_[kWave] + po_[2 * kWave] + po_[3 * kWave];
+      }
+      const float* pk_ = part_k + buf * 4 * kWave + lane;
+      const float ks = pk_[0] + pk_[kWave] + pk_[2 * kWave] + pk_[3 * kWave];
+      const float u = beta * (vv - dec * ks);       // the state is decayed before it is read
+      float po4[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+      for (int r = 0; r < DR; ++r) {
+        s[r] = dec * s[r] + kr[r] * u;
+        po4[r & 3] += s[r] * qr[r];
+      }
+      part_o[(buf * 4 + rp) * kWave + lane] = (po4[0] + po4[1]) + (po4[2] + po4[3]);
     }
-    part_o[buf][rp][lane] = po;
-  }
-  __syncthreads();
-  {
-    const int pb = (n - 1) & 1;
-    if (rp == 0 && live)
-      p.o[((static_cast<int64_t>(q0) + n - 1) * p.H + h) * p.Dv + col] =
-          part_o[pb][0][lane] + part_o[pb][1][lane] + part_o[pb][2][lane] + part_o[pb][3][lane];
+    __syncthreads();
+    if (rp == 0) {                                  // the chunk's last token
+      const float* po_ = part_o + ((cn - 1) & 1) * 4 * kWave + lane;
+      o_lds[(cn - 1) * kWave + lane] = po_[0] + po_[kWave] + po_[2 * kWave] + po_[3 * kWave];
+    }
+    __syncthreads();
+    for (int x = threadIdx.x; x < cn * kWave; x += blockDim.x) {
+      const int tok = x / kWave, cc = blockIdx.x * kWave + (x % kWave);
+      if (cc < p.Dv) p.o[((static_cast<int64_t>(q0) + c0 + tok) * p.H + h) * p.Dv + cc] = o_lds[x];
+    }
   }
   if (live) {
 #pragma unroll
     for (int r = 0; r < DR; ++r)
       if (row0 + r < p.D) sbase[static_cast<int64_t>(row0 + r) * p.Dv + col] = s[r];
   }
+}
+
+template <int DR>
+static void delta_rule_launch(const DeltaRuleParams& p, dim3 grid, hipStream_t s) {
+  const size_t shm = sizeof(float) * (2 * kDeltaChunk * 4 * DR + 2 * kDeltaChunk * kWave + kDeltaChunk * 2 + 4 * 4 * kWave);
+  gated_delta_rule_kernel<DR><<<grid, dim3(256), shm, s>>>(p);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -357,7 +429,12 @@ int lv_clamped_glu(const void* in, int64_t ld_in, void* out, int64_t T, int F, f
   if (in == nullptr || out == nullptr || T < 0 || F <= 0 || ld_in < 2 * F) return fail(-1, "lv_clamped_glu: bad arguments");
   const int64_t n = T * F;
   dim3 grid(static_cast<unsigned>((n + 255) / 256)), block(256);
-  if (dtype == LV_MIX_BF16)
+  if (dtype == LV_MIX_BF16 && F % 8 == 0 && ld_in % 8 == 0 && (reinterpret_cast<uintptr_t>(in) & 15) == 0 &&
+      (reinterpret_cast<uintptr_t>(out) & 15) == 0) {
+    dim3 grid8(static_cast<unsigned>((n / 8 + 255) / 256));
+    clamped_glu_bf16x8_kernel<<<grid8, block, 0, as_stream(stream)>>>(static_cast<const uint16_t*>(in), ld_in,
+                                                                     static_cast<uint16_t*>(out), T, F / 8, limit, alpha);
+  } else if (dtype == LV_MIX_BF16)
     clamped_glu_kernel<bf16_t><<<grid, block, 0, as_stream(stream)>>>(static_cast<const bf16_t*>(in), ld_in,
                                                                     static_cast<bf16_t*>(out), T, F, limit, alpha);
   else if (dtype == LV_MIX_F32)
@@ -419,12 +496,12 @@ int lv_gated_delta_rule(const void* qn, const void* kn, const void* v, const voi
   DeltaRuleParams p{static_cast<const float*>(qn), static_cast<const float*>(kn), static_cast<const float*>(v),
                     static_cast<const float*>(beta), static_cast<const float*>(decay), static_cast<float*>(state),
                     cu_q, ctx_lens, slots, static_cast<float*>(o), G, H, D, Dv};
-  dim3 grid((Dv + kWave - 1) / kWave, H, B), block(256);
+  dim3 grid((Dv + kWave - 1) / kWave, H, B);
   hipStream_t s = as_stream(stream);
-  if (D <= 32) gated_delta_rule_kernel<8><<<grid, block, 0, s>>>(p);
-  else if (D <= 64) gated_delta_rule_kernel<16><<<grid, block, 0, s>>>(p);
-  else if (D <= 128) gated_delta_rule_kernel<32><<<grid, block, 0, s>>>(p);
-  else gated_delta_rule_kernel<64><<<grid, block, 0, s>>>(p);
+  if (D <= 32) delta_rule_launch<8>(p, grid, s);
+  else if (D <= 64) delta_rule_launch<16>(p, grid, s);
+  else if (D <= 128) delta_rule_launch<32>(p, grid, s);
+  else delta_rule_launch<64>(p, grid, s);
   return launched("lv_gated_delta_rule");
 }
 

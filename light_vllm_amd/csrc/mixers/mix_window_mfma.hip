@@ -6,17 +6,20 @@
 // query does not see (outside its window, a block not yet wholly before it, the future) is masked.
 //
 // Everything is computed transposed so that no operand changes layout between the two products:
-//   S^T = K Q^T   v_mfma_f32_16x16x16_bf16, A = 16 keys x 16 of D read straight from the cache rows,
-//                 B = the wave's Q fragments (registers, loaded once); a lane ends up with 4 keys of ONE query,
-//                 so the softmax statistics of a query live in 4 lanes (two shuffles) and
-//   O^T += V^T P^T  takes the probabilities as its B operand exactly as they lie (keys x queries), with
-//                 A = V^T read from the 64-entry V tile that the four waves stage in LDS together.
+//   S^T = K Q^T   v_mfma_f32_16x16x32_bf16 (one 16x16x16 step more when D is an odd multiple of 16), A = 16 keys x 32
+//                 of D read straight from the cache rows with 16-byte loads, B = the wave's Q fragments (registers,
+//                 loaded once); a lane ends up with 4 keys of ONE query, so the softmax statistics of a query live
+//                 in 4 lanes (two shuffles) and
+//   O^T += V^T P^T  takes the probabilities of two 16-key blocks as its B operand exactly as they lie (keys x
+//                 queries), with A = V^T read as two 8-byte runs of keys from the 64-entry V tile that the four
+//                 waves stage TRANSPOSED in LDS together.
 // The sink is the initial state of the running softmax: maximum 0, sum 1.
 #include "mix_common.h"
 
 namespace lvmix {
 
 typedef __attribute__((ext_vector_type(4))) short bf16x4_t;
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
 typedef __attribute__((ext_vector_type(4))) float f32x4_t;
 
 struct WindowMfmaParams {
@@ -30,7 +33,8 @@ struct WindowMfmaParams {
 
 constexpr int kTileQ = 16;
 constexpr int kTileK = 64;
-constexpr int kMaxKK = 16;     // D <= 256
+constexpr int kMaxK32 = 8;     // D <= 256: 32-wide steps over D, plus one 16-wide when D % 32 == 16
+constexpr int kLdk = kTileK + 4; // row stride (in keys) of the transposed V tile: rows stay 8-byte aligned
 constexpr int kMaxDvb = 16;    // Dv <= 256
 
 __device__ __forceinline__ short bf16_bits(float x) {
@@ -38,8 +42,12 @@ __device__ __forceinline__ short bf16_bits(float x) {
   return __builtin_bit_cast(short, b);
 }
 
+// AHEAD: fetch the next tile's V rows and key-row addresses while the current tile is computed. It pays when a
+// launch has few workgroups per compute unit (single decoded tokens); a prompt's many tiles hide latency by
+// occupancy, which the extra registers would cost.
+template <bool AHEAD>
 __global__ __launch_bounds__(256) void window_pool_mfma_kernel(WindowMfmaParams p) {
-  extern __shared__ uint16_t vs[];                      // [kTileK][Dv + 4]
+  extern __shared__ uint16_t vs[];                      // V^T tile [Dv][kLdk]
   const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
   const int ln = lane & 15, lg = lane >> 4;
   const int b = blockIdx.z;
@@ -59,16 +67,19 @@ __global__ __launch_bounds__(256) void window_pool_mfma_kernel(WindowMfmaParams 
   const bool active = hloc < rep;
   const int h = g * rep + min(hloc, rep - 1);
   const int D = p.D, Dv = p.Dv, page = p.page, P = p.P, W = p.window;
-  const int nkk = D / 16, ndvb = Dv / 16, ldv = Dv + 4;
+  const int nk32 = D / 32, ndvb = Dv / 16;
+  const bool tail16 = (D & 16) != 0;
   const int64_t GD = static_cast<int64_t>(p.G) * D, GDv = static_cast<int64_t>(p.G) * Dv;
   const int32_t* bt = p.block_tables + static_cast<int64_t>(b) * p.bt_stride;
 
-  bf16x4_t qf[kMaxKK];
+  bf16x8_t qf[kMaxK32];
+  bf16x4_t qtail = bf16x4_t{0, 0, 0, 0};
   {
-    const uint16_t* qrow = p.q + (t * p.H + h) * D + 4 * lg;
+    const uint16_t* qrow = p.q + (t * p.H + h) * D;
 #pragma unroll
-    for (int kk = 0; kk < kMaxKK; ++kk)
-      if (kk < nkk) qf[kk] = *reinterpret_cast<const bf16x4_t*>(qrow + 16 * kk);
+    for (int kk = 0; kk < kMaxK32; ++kk)
+      if (kk < nk32) qf[kk] = *reinterpret_cast<const bf16x8_t*>(qrow + 32 * kk + 8 * lg);
+    if (tail16) qtail = *reinterpret_cast<const bf16x4_t*>(qrow + 32 * nk32 + 4 * lg);
   }
   f32x4_t acc_o[kMaxDvb];
 #pragma unroll
@@ -78,44 +89,104 @@ __global__ __launch_bounds__(256) void window_pool_mfma_kernel(WindowMfmaParams 
   const int nbmax = (P > 0 && i1 - W + 1 > 0) ? (i1 - W + 1) / P : 0;      // pooled blocks the last query sees
   const int jlo = max(0, i0 - W + 1);
 
-  for (int phase = 0; phase < 2; ++phase) {
-    const int e_begin = phase == 0 ? 0 : jlo;
-    const int e_end = phase == 0 ? nbmax : i1 + 1;                          // entries [e_begin, e_end)
-    for (int e0 = e_begin; e0 < e_end; e0 += kTileK) {
-      __syncthreads();                                                      // the previous tile's V reads are done
-      for (int c = threadIdx.x; c < kTileK * (Dv / 4); c += blockDim.x) {
-        const int row = c / (Dv / 4), seg = c - row * (Dv / 4);
-        const int e = min(e0 + row, e_end - 1);
-        const uint16_t* vrow;
-        if (phase == 0) {
-          const int pj = (e * P + P - 1) / page;
-          vrow = p.vp + (static_cast<int64_t>(bt[pj]) * p.PP + (e - (page * pj) / P)) * GDv + g * Dv;
-        } else {
-          vrow = p.v_cache + (static_cast<int64_t>(bt[e / page]) * page + e % page) * GDv + g * Dv;
-        }
-        *reinterpret_cast<uint2*>(vs + row * ldv + seg * 4) = *reinterpret_cast<const uint2*>(vrow + seg * 4);
-      }
-      __syncthreads();
-      if (!active) continue;
+  // The tiles of both phases as one list: [pooled tiles | token tiles]. The V rows of the next tile and the
+  // addresses of its key rows are fetched while the current tile is computed; they meet LDS behind a barrier.
+  const int npt = (nbmax + kTileK - 1) / kTileK;
+  const int ntt = (i1 + 1 - jlo + kTileK - 1) / kTileK;
+  const int ntiles = npt + ntt;
+  const int vrow_id = threadIdx.x >> 2, vq = threadIdx.x & 3;             // staging: 4 threads per V row
+  const int nseg = Dv / 4;                                                // 8-byte segments of a row
 
+  auto entry_rows = [&](int tile, int e, const uint16_t*& kr_, const uint16_t*& vr_) {
+    if (tile < npt) {
+      const int ec = min(e, nbmax - 1);
+      const int pj = (ec * P + P - 1) / page;
+      const int64_t slot = static_cast<int64_t>(bt[pj]) * p.PP + (ec - (page * pj) / P);
+      kr_ = p.kp + slot * GD + g * D;
+      vr_ = p.vp + slot * GDv + g * Dv;
+    } else {
+      const int ec = min(e, i1);
+      const int64_t slot = static_cast<int64_t>(bt[ec / page]) * page + ec % page;
+      kr_ = p.k_cache + slot * GD + g * D;
+      vr_ = p.v_cache + slot * GDv + g * Dv;
+    }
+  };
+  auto tile_start = [&](int tile) { return tile < npt ? tile * kTileK : jlo + (tile - npt) * kTileK; };
+
+  uint2 vreg[kMaxDvb];
+  const uint16_t* knext[4];
+  auto prefetch = [&](int tile) {
+    const int e0 = tile_start(tile);
+    const uint16_t *kr_, *vr_;
+    entry_rows(tile, e0 + vrow_id, kr_, vr_);
+#pragma unroll
+    for (int x = 0; x < kMaxDvb; ++x) {
+      const int seg = vq + 4 * x;
+      if (seg < nseg) vreg[x] = *reinterpret_cast<const uint2*>(vr_ + seg * 4);
+    }
+#pragma unroll
+    for (int kb = 0; kb < 4; ++kb) {
+      const uint16_t* unused;
+      entry_rows(tile, e0 + kb * 16 + ln, knext[kb], unused);
+    }
+  };
+  if (AHEAD && ntiles > 0) prefetch(0);
+  for (int tile = 0; tile < ntiles; ++tile) {
+    const int phase = tile < npt ? 0 : 1;
+    const int e0 = tile_start(tile);
+    const int e_end = phase == 0 ? nbmax : i1 + 1;
+    const uint16_t* kcur[4];
+    __syncthreads();                                                        // the previous tile's V reads are done
+    if (AHEAD) {
+#pragma unroll
+      for (int x = 0; x < kMaxDvb; ++x) {
+        const int seg = vq + 4 * x;
+        if (seg < nseg) {
+          uint16_t* dst = vs + (seg * 4) * kLdk + vrow_id;
+          dst[0] = static_cast<uint16_t>(vreg[x].x & 0xffffu);
+          dst[kLdk] = static_cast<uint16_t>(vreg[x].x >> 16);
+          dst[2 * kLdk] = static_cast<uint16_t>(vreg[x].y & 0xffffu);
+          dst[3 * kLdk] = static_cast<uint16_t>(vreg[x].y >> 16);
+        }
+      }
+#pragma unroll
+      for (int kb = 0; kb < 4; ++kb) kcur[kb] = knext[kb];
+    } else {
+      // consecutive threads take consecutive 8-byte segments of a row: whole cache lines per load instruction
+      for (int c = threadIdx.x; c < kTileK * nseg; c += blockDim.x) {
+        const int row = c / nseg, seg = c - row * nseg;
+        const uint16_t *kr_, *vr_;
+        entry_rows(tile, e0 + row, kr_, vr_);
+        const uint2 v4 = *reinterpret_cast<const uint2*>(vr_ + seg * 4);
+        uint16_t* dst = vs + (seg * 4) * kLdk + row;
+        dst[0] = static_cast<uint16_t>(v4.x & 0xffffu);
+        dst[kLdk] = static_cast<uint16_t>(v4.x >> 16);
+        dst[2 * kLdk] = static_cast<uint16_t>(v4.y & 0xffffu);
+        dst[3 * kLdk] = static_cast<uint16_t>(v4.y >> 16);
+      }
+#pragma unroll
+      for (int kb = 0; kb < 4; ++kb) {
+        const uint16_t* unused;
+        entry_rows(tile, e0 + kb * 16 + ln, kcur[kb], unused);
+      }
+    }
+    __syncthreads();
+    if (AHEAD && tile + 1 < ntiles) prefetch(tile + 1);
+    if (!active) continue;
+    {
       float s[4][4];
 #pragma unroll
       for (int kb = 0; kb < 4; ++kb) {
-        const int e = min(e0 + kb * 16 + ln, e_end - 1);                    // this lane's A row: one key
-        const uint16_t* krow;
-        if (phase == 0) {
-          const int pj = (e * P + P - 1) / page;
-          krow = p.kp + (static_cast<int64_t>(bt[pj]) * p.PP + (e - (page * pj) / P)) * GD + g * D;
-        } else {
-          krow = p.k_cache + (static_cast<int64_t>(bt[e / page]) * page + e % page) * GD + g * D;
-        }
-        krow += 4 * lg;
+        const uint16_t* krow = kcur[kb];
         f32x4_t acc = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-        for (int kk = 0; kk < kMaxKK; ++kk)
-          if (kk < nkk)
-            acc = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(*reinterpret_cast<const bf16x4_t*>(krow + 16 * kk), qf[kk],
-                                                            acc, 0, 0, 0);
+        for (int kk = 0; kk < kMaxK32; ++kk)
+          if (kk < nk32)
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*reinterpret_cast<const bf16x8_t*>(krow + 32 * kk + 8 * lg),
+                                                          qf[kk], acc, 0, 0, 0);
+        if (tail16)
+          acc = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(*reinterpret_cast<const bf16x4_t*>(krow + 32 * nk32 + 4 * lg),
+                                                          qtail, acc, 0, 0, 0);
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           const int ke = e0 + kb * 16 + 4 * lg + i;                         // the key of result row 4*lg + i
@@ -135,14 +206,14 @@ __global__ __launch_bounds__(256) void window_pool_mfma_kernel(WindowMfmaParams 
       const float nm = fmaxf(m, mx);
       const float corr = expf(m - nm);
       float rs = 0.0f;
-      bf16x4_t pb[4];
+      bf16x8_t pb[2];                                                       // key blocks (0, 1) and (2, 3) side by side
 #pragma unroll
       for (int kb = 0; kb < 4; ++kb) {
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           const float e = expf(s[kb][i] - nm);                              // exp(-inf) = 0 for what is not seen
           rs += e;
-          pb[kb][i] = bf16_bits(e);
+          pb[kb >> 1][(kb & 1) * 4 + i] = static_cast<__bf16>(e);
         }
       }
       rs += __shfl_xor(rs, 16, kWave);
@@ -153,15 +224,15 @@ __global__ __launch_bounds__(256) void window_pool_mfma_kernel(WindowMfmaParams 
       for (int d = 0; d < kMaxDvb; ++d)
         if (d < ndvb) acc_o[d] *= corr;
 #pragma unroll
-      for (int kb = 0; kb < 4; ++kb) {
-        const uint16_t* vt = vs + (kb * 16 + 4 * lg) * ldv + ln;            // V^T fragment: 4 keys of one value column
+      for (int c = 0; c < 2; ++c) {
+        const uint16_t* vt = vs + ln * kLdk + c * 32 + 4 * lg;              // value column ln: keys 4lg.. of blocks 2c, 2c+1
 #pragma unroll
         for (int d = 0; d < kMaxDvb; ++d) {
           if (d < ndvb) {
-            bf16x4_t a;
-#pragma unroll
-            for (int i = 0; i < 4; ++i) a[i] = static_cast<short>(vt[i * ldv + 16 * d]);
-            acc_o[d] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, pb[kb], acc_o[d], 0, 0, 0);
+            const uint2 lo = *reinterpret_cast<const uint2*>(vt + 16 * d * kLdk);
+            const uint2 hi = *reinterpret_cast<const uint2*>(vt + 16 * d * kLdk + 16);
+            const uint4 both = uint4{lo.x, lo.y, hi.x, hi.y};
+            acc_o[d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, both), pb[c], acc_o[d], 0, 0, 0);
           }
         }
       }
@@ -200,7 +271,7 @@ extern "C" int lv_window_pool_attn_mfma(const void* q, const void* k_cache, cons
   if (P > 0 && (!kp || !vp)) return fail(-1, "lv_window_pool_attn_mfma: pooled blocks without their cache");
   if (B < 0 || H <= 0 || G <= 0 || H % G != 0 || page <= 0 || window <= 0 || bt_stride <= 0)
     return fail(-1, "lv_window_pool_attn_mfma: bad sizes");
-  if (D % 16 != 0 || Dv % 16 != 0 || D <= 0 || Dv <= 0 || D > 16 * kMaxKK || Dv > 16 * kMaxDvb)
+  if (D % 16 != 0 || Dv % 16 != 0 || D <= 0 || Dv <= 0 || D > 32 * kMaxK32 || Dv > 16 * kMaxDvb)
     return fail(-2, "lv_window_pool_attn_mfma: head sizes %d / %d (multiples of 16 up to 256)", D, Dv);
   if (gate != nullptr && ld_gate < static_cast<int64_t>(H) * Dv) return fail(-1, "lv_window_pool_attn_mfma: gate stride");
   const int rep = H / G;
@@ -210,8 +281,9 @@ extern "C" int lv_window_pool_attn_mfma(const void* q, const void* k_cache, cons
                      static_cast<const uint16_t*>(vp), static_cast<const uint16_t*>(gate), ld_gate,
                      static_cast<uint16_t*>(out), cu_q, ctx_lens, block_tables, bt_stride, H, G, D, Dv, page, window, P,
                      P > 0 ? (page + P - 1) / P : 0, ngroups, scale, has_sink ? 1.0f : 0.0f};
-  const size_t shm = static_cast<size_t>(kTileK) * (Dv + 4) * sizeof(uint16_t);
+  const size_t shm = static_cast<size_t>(Dv) * kLdk * sizeof(uint16_t);
   dim3 grid((max_new_tokens + kTileQ - 1) / kTileQ, G * ngroups, B), block(256);
-  window_pool_mfma_kernel<<<grid, block, shm, as_stream(stream)>>>(p);
+  if (max_new_tokens <= kTileQ) window_pool_mfma_kernel<true><<<grid, block, shm, as_stream(stream)>>>(p);
+  else window_pool_mfma_kernel<false><<<grid, block, shm, as_stream(stream)>>>(p);
   return launched("lv_window_pool_attn_mfma");
 }
