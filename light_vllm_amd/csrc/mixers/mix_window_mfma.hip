@@ -33,19 +33,20 @@ struct WindowMfmaParams {
 
 constexpr int kTileQ = 16;
 constexpr int kTileK = 64;
-constexpr int kMaxK32 = 8;     // D <= 256: 32-wide steps over D, plus one 16-wide when D % 32 == 16
+constexpr int kMaxK32 = 8;     // D <= 256: 32-wide steps over D (template K32: 4 up to D = 128), plus one 16-wide when D % 32 == 16
 constexpr int kLdk = kTileK + 4; // row stride (in keys) of the transposed V tile: rows stay 8-byte aligned
 constexpr int kMaxDvb = 16;    // Dv <= 256
+constexpr int kBtCache = 2048; // page ids of a sequence kept in LDS (longer sequences look them up in memory)
 
 __device__ __forceinline__ short bf16_bits(float x) {
   __bf16 b = static_cast<__bf16>(x);
   return __builtin_bit_cast(short, b);
 }
 
-// AHEAD: fetch the next tile's V rows and key-row addresses while the current tile is computed. It pays when a
-// launch has few workgroups per compute unit (single decoded tokens); a prompt's many tiles hide latency by
-// occupancy, which the extra registers would cost.
-template <bool AHEAD>
+// AHEAD: fetch the next tile's V rows, key-row addresses and (once the current scores are done) K fragments while
+// the current tile is computed. It pays when a launch has few workgroups per compute unit (single decoded tokens); a
+// prompt's many tiles hide latency by occupancy, which the extra registers would cost.
+template <bool AHEAD, int K32>
 __global__ __launch_bounds__(256) void window_pool_mfma_kernel(WindowMfmaParams p) {
   extern __shared__ uint16_t vs[];                      // V^T tile [Dv][kLdk]
   const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
@@ -70,14 +71,23 @@ __global__ __launch_bounds__(256) void window_pool_mfma_kernel(WindowMfmaParams 
   const int nk32 = D / 32, ndvb = Dv / 16;
   const bool tail16 = (D & 16) != 0;
   const int64_t GD = static_cast<int64_t>(p.G) * D, GDv = static_cast<int64_t>(p.G) * Dv;
-  const int32_t* bt = p.block_tables + static_cast<int64_t>(b) * p.bt_stride;
+  const int32_t* bt_global = p.block_tables + static_cast<int64_t>(b) * p.bt_stride;
+  // the sequence's page ids up to the last query's page, once, so that no row address waits for a second trip to memory
+  __shared__ int32_t bt_lds[kBtCache];
+  const int nbt = (ctx + r0 + nvalid - 1) / page + 1;
+  const bool bt_cached = nbt <= kBtCache;
+  if (bt_cached) {
+    for (int x = threadIdx.x; x < nbt; x += blockDim.x) bt_lds[x] = bt_global[x];
+    __syncthreads();
+  }
+  auto bt = [&](int idx) { return bt_cached ? bt_lds[idx] : bt_global[idx]; };
 
-  bf16x8_t qf[kMaxK32];
+  bf16x8_t qf[K32];
   bf16x4_t qtail = bf16x4_t{0, 0, 0, 0};
   {
     const uint16_t* qrow = p.q + (t * p.H + h) * D;
 #pragma unroll
-    for (int kk = 0; kk < kMaxK32; ++kk)
+    for (int kk = 0; kk < K32; ++kk)
       if (kk < nk32) qf[kk] = *reinterpret_cast<const bf16x8_t*>(qrow + 32 * kk + 8 * lg);
     if (tail16) qtail = *reinterpret_cast<const bf16x4_t*>(qrow + 32 * nk32 + 4 * lg);
   }
@@ -101,12 +111,12 @@ __global__ __launch_bounds__(256) void window_pool_mfma_kernel(WindowMfmaParams 
     if (tile < npt) {
       const int ec = min(e, nbmax - 1);
       const int pj = (ec * P + P - 1) / page;
-      const int64_t slot = static_cast<int64_t>(bt[pj]) * p.PP + (ec - (page * pj) / P);
+      const int64_t slot = static_cast<int64_t>(bt(pj)) * p.PP + (ec - (page * pj) / P);
       kr_ = p.kp + slot * GD + g * D;
       vr_ = p.vp + slot * GDv + g * Dv;
     } else {
       const int ec = min(e, i1);
-      const int64_t slot = static_cast<int64_t>(bt[ec / page]) * page + ec % page;
+      const int64_t slot = static_cast<int64_t>(bt(ec / page)) * page + ec % page;
       kr_ = p.k_cache + slot * GD + g * D;
       vr_ = p.v_cache + slot * GDv + g * Dv;
     }
@@ -130,13 +140,33 @@ __global__ __launch_bounds__(256) void window_pool_mfma_kernel(WindowMfmaParams 
       entry_rows(tile, e0 + kb * 16 + ln, knext[kb], unused);
     }
   };
-  if (AHEAD && ntiles > 0) prefetch(0);
+  // Only LDS traffic meets at the barriers of the tile loop. The fetch-ahead variant waits for that alone, so the
+  // vector loads of the next tile stay in flight across them (a full __syncthreads would drain them every tile).
+  auto tile_barrier = [&]() {
+    if (AHEAD) asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    else __syncthreads();
+  };
+  bf16x8_t kdata[4][K32];
+  bf16x4_t ktail[4];
+  auto fetch_k = [&]() {                                                    // the K fragments of the tile knext points to
+#pragma unroll
+    for (int kb = 0; kb < 4; ++kb) {
+#pragma unroll
+      for (int kk = 0; kk < K32; ++kk)
+        if (kk < nk32) kdata[kb][kk] = *reinterpret_cast<const bf16x8_t*>(knext[kb] + 32 * kk + 8 * lg);
+      if (tail16) ktail[kb] = *reinterpret_cast<const bf16x4_t*>(knext[kb] + 32 * nk32 + 4 * lg);
+    }
+  };
+  if (AHEAD && ntiles > 0) {
+    prefetch(0);
+    if (active) fetch_k();
+  }
   for (int tile = 0; tile < ntiles; ++tile) {
     const int phase = tile < npt ? 0 : 1;
     const int e0 = tile_start(tile);
     const int e_end = phase == 0 ? nbmax : i1 + 1;
     const uint16_t* kcur[4];
-    __syncthreads();                                                        // the previous tile's V reads are done
+    tile_barrier();                                                         // the previous tile's V reads are done
     if (AHEAD) {
 #pragma unroll
       for (int x = 0; x < kMaxDvb; ++x) {
@@ -170,7 +200,7 @@ __global__ __launch_bounds__(256) void window_pool_mfma_kernel(WindowMfmaParams 
         entry_rows(tile, e0 + kb * 16 + ln, kcur[kb], unused);
       }
     }
-    __syncthreads();
+    tile_barrier();
     if (AHEAD && tile + 1 < ntiles) prefetch(tile + 1);
     if (!active) continue;
     {
@@ -180,13 +210,13 @@ __global__ __launch_bounds__(256) void window_pool_mfma_kernel(WindowMfmaParams 
         const uint16_t* krow = kcur[kb];
         f32x4_t acc = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-        for (int kk = 0; kk < kMaxK32; ++kk)
+        for (int kk = 0; kk < K32; ++kk)
           if (kk < nk32)
-            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*reinterpret_cast<const bf16x8_t*>(krow + 32 * kk + 8 * lg),
-                                                          qf[kk], acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                AHEAD ? kdata[kb][kk] : *reinterpret_cast<const bf16x8_t*>(krow + 32 * kk + 8 * lg), qf[kk], acc, 0, 0, 0);
         if (tail16)
-          acc = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(*reinterpret_cast<const bf16x4_t*>(krow + 32 * nk32 + 4 * lg),
-                                                          qtail, acc, 0, 0, 0);
+          acc = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(
+              AHEAD ? ktail[kb] : *reinterpret_cast<const bf16x4_t*>(krow + 32 * nk32 + 4 * lg), qtail, acc, 0, 0, 0);
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           const int ke = e0 + kb * 16 + 4 * lg + i;                         // the key of result row 4*lg + i
@@ -196,6 +226,7 @@ __global__ __launch_bounds__(256) void window_pool_mfma_kernel(WindowMfmaParams 
           s[kb][i] = vis ? acc[i] * p.scale : -INFINITY;
         }
       }
+      if (AHEAD && tile + 1 < ntiles) fetch_k();                            // in flight across the softmax, PV and the barriers
       float mx = -INFINITY;
 #pragma unroll
       for (int kb = 0; kb < 4; ++kb)
@@ -283,7 +314,13 @@ extern "C" int lv_window_pool_attn_mfma(const void* q, const void* k_cache, cons
                      P > 0 ? (page + P - 1) / P : 0, ngroups, scale, has_sink ? 1.0f : 0.0f};
   const size_t shm = static_cast<size_t>(Dv) * kLdk * sizeof(uint16_t);
   dim3 grid((max_new_tokens + kTileQ - 1) / kTileQ, G * ngroups, B), block(256);
-  if (max_new_tokens <= kTileQ) window_pool_mfma_kernel<true><<<grid, block, shm, as_stream(stream)>>>(p);
-  else window_pool_mfma_kernel<false><<<grid, block, shm, as_stream(stream)>>>(p);
+  hipStream_t st = as_stream(stream);
+  if (max_new_tokens <= kTileQ) {
+    if (D <= 128) window_pool_mfma_kernel<true, 4><<<grid, block, shm, st>>>(p);
+    else window_pool_mfma_kernel<true, kMaxK32><<<grid, block, shm, st>>>(p);
+  } else {
+    if (D <= 128) window_pool_mfma_kernel<false, 4><<<grid, block, shm, st>>>(p);
+    else window_pool_mfma_kernel<false, kMaxK32><<<grid, block, shm, st>>>(p);
+  }
   return launched("lv_window_pool_attn_mfma");
 }

@@ -326,3 +326,28 @@ def case_generate(device, tmp_path):
             assert (top2[0] - top2[1]).item() > 2e-4 * logits.abs().max().item(), "oracle tie: pick another seed"
             seq.append(int(logits.argmax()))
         assert out["token_ids"] == seq[len(p):]
+
+
+def case_generate_preemption(device, tmp_path):
+    """A page pool too small for the sequences that run: the scheduler preempts from the tail, frees pages and
+    state slot, and recomputes the preempted sequence from its first token later; completions do not change."""
+    from light_vllm_amd.llm import LLM
+    from light_vllm_amd.sampling_params import SamplingParams
+    cfg = K.CFG_MAIN
+    model_dir, weights = _model(tmp_path, cfg, 8)
+    prompts = [K.tokens_for(cfg, n, 50 + n) for n in (27, 29, 14)]
+    steps = 9
+    llm = LLM(model_dir, dtype="float32", device=device, kvcache_block_size=16, max_num_seqs=3, max_cache_tokens=64,
+              max_num_batched_tokens=32, max_model_len=64)
+    preempted = []
+    original = llm.scheduler.preempt
+    llm.scheduler.preempt = lambda seq: (preempted.append(seq.seq_id), original(seq))[1]
+    outs = llm.generate([list(p) for p in prompts], SamplingParams(temperature=0.0, max_tokens=steps, ignore_eos=True))
+    assert preempted, "the case is meant to run out of pages"
+    assert llm.scheduler.block_manager.num_free_blocks == 4 and llm.scheduler.state_slots.num_free == 3
+    llm.exit()
+    for p, out in zip(prompts, outs):
+        seq = list(p)
+        for _ in range(steps):
+            seq.append(int(oracle.forward(cfg, weights, seq)[-1].argmax()))
+        assert out["token_ids"] == seq[len(p):]

@@ -50,6 +50,10 @@ def test_generate_greedy(tmp_path):
     C.case_generate(DEV, tmp_path)
 
 
+def test_generate_under_preemption(tmp_path):
+    C.case_generate_preemption(DEV, tmp_path)
+
+
 def test_config_reader_rejects_what_it_does_not_know():
     from light_vllm_amd.models.kagalorn import KagalornConfig
     good = {k: v for k, v in K.CFG_MAIN.items()}

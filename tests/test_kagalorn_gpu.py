@@ -65,3 +65,7 @@ def test_engine_long_decode(gpu, tmp_path):
 
 def test_generate_greedy(gpu, tmp_path):
     C.case_generate(DEV, tmp_path)
+
+
+def test_generate_under_preemption(gpu, tmp_path):
+    C.case_generate_preemption(DEV, tmp_path)
