@@ -782,7 +782,7 @@ def main():
     ap.add_argument("--rehearse", action="store_true",
                     help="N > 1 on ONE GPU: every rank on cuda:0, gloo group, 4 layers, batch 8 "
                          "(proves launcher, rendezvous, graph and JSON path; not a measurement)")
-    ap.add_argument("--mixers", default="", help="comma list of sizes (2k, 4k): instead of the contract workload, "
+    ap.add_argument("--mixers", default="", help="comma list of sizes (2k, 4k): instead of the default workload, "
                     "run the Kagalorn design beside Qwen3 at equal size and time its kernels one by one")
     ap.add_argument("--mixers-batch", type=int, default=16)
     ap.add_argument("--mixers-prompt", type=int, default=1024)

@@ -35,7 +35,7 @@
 extern "C" {
 #endif
 
-#define LV_MIX_ABI_VERSION 3
+#define LV_MIX_ABI_VERSION 4
 #define LV_MIX_BF16 0
 #define LV_MIX_F32 1
 #define LV_MIX_MAX_STREAMS 8
@@ -104,11 +104,14 @@ int lv_window_pool_attn(const void* q, const void* k_cache, const void* v_cache,
                         void* stream);
 
 /* The same attention on the matrix cores: bf16 only, D and Dv multiples of 16 up to 256. Tiles of 16 new
- * tokens per sequence; max_new_tokens = the largest cu_q[b+1] - cu_q[b] of the step. */
+ * tokens per sequence; max_new_tokens = the largest cu_q[b+1] - cu_q[b] of the step.
+ * nsplit > 1 (only with max_new_tokens <= 16, i.e. decode-shaped steps): the key tiles of a sequence are cut over nsplit
+ * workgroups whose partials a second kernel merges; workspace: f32 [T, H, nsplit, Dv + 4] (read-out, maximum, sum, padding), T = total new tokens. */
 int lv_window_pool_attn_mfma(const void* q, const void* k_cache, const void* v_cache, const void* kp, const void* vp,
                              const void* gate, int64_t ld_gate, void* out, const int32_t* cu_q, const int32_t* ctx_lens,
                              const int32_t* block_tables, int bt_stride, int B, int max_new_tokens, int H, int G, int D,
-                             int Dv, int page, int window, int P, float scale, int has_sink, void* stream);
+                             int Dv, int page, int window, int P, float scale, int has_sink, int nsplit, void* workspace,
+                             int64_t T, void* stream);
 
 #ifdef __cplusplus
 }

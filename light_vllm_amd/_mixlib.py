@@ -16,7 +16,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(_HERE, "csrc", "mixers")
 LIB_PATH = os.path.join(_HERE, "lib", "liblvmix.so")
 SOURCES = ["mix_stream.hip", "mix_window_attn.hip", "mix_window_mfma.hip"]
-ABI_VERSION = 3
+ABI_VERSION = 4
 
 _P = c_void_p
 SIGNATURES = {
@@ -36,7 +36,7 @@ SIGNATURES = {
     "lv_window_pool_attn": (c_int, [_P, _P, _P, _P, _P, _P, c_int64, _P, _P, _P, _P, _P, c_int, c_int64, c_int,
                                     c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, _P]),
     "lv_window_pool_attn_mfma": (c_int, [_P, _P, _P, _P, _P, _P, c_int64, _P, _P, _P, _P, c_int, c_int, c_int, c_int,
-                                         c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, _P]),
+                                         c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, _P, c_int64, _P]),
 }
 
 _lib = None

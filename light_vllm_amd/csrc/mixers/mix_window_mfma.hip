@@ -29,6 +29,8 @@ struct WindowMfmaParams {
   const int32_t *cu_q, *ctx_lens, *block_tables;
   int bt_stride, H, G, D, Dv, page, window, P, PP, ngroups;
   float scale, sink;
+  int nsplit;          // > 1 (launches of at most one query tile per sequence): grid.x = split of the key tiles
+  float* ws;           // [T, H, nsplit, Dv + 4] partial read-outs, running maximum and sum
 };
 
 constexpr int kTileQ = 16;
@@ -54,7 +56,8 @@ __global__ __launch_bounds__(256) void window_pool_mfma_kernel(WindowMfmaParams 
   const int b = blockIdx.z;
   const int g = blockIdx.y / p.ngroups, hg = blockIdx.y % p.ngroups;
   const int q0 = p.cu_q[b], n = p.cu_q[b + 1] - q0;
-  const int r0 = blockIdx.x * kTileQ;
+  const int split = p.nsplit > 1 ? blockIdx.x : 0;
+  const int r0 = p.nsplit > 1 ? 0 : blockIdx.x * kTileQ;
   if (r0 >= n) return;
   const int ctx = p.ctx_lens[b];
   const int nvalid = min(kTileQ, n - r0);
@@ -94,7 +97,7 @@ __global__ __launch_bounds__(256) void window_pool_mfma_kernel(WindowMfmaParams 
   f32x4_t acc_o[kMaxDvb];
 #pragma unroll
   for (int d = 0; d < kMaxDvb; ++d) acc_o[d] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
-  float m = 0.0f, l = p.sink;
+  float m = 0.0f, l = split == 0 ? p.sink : 0.0f;
 
   const int nbmax = (P > 0 && i1 - W + 1 > 0) ? (i1 - W + 1) / P : 0;      // pooled blocks the last query sees
   const int jlo = max(0, i0 - W + 1);
@@ -157,11 +160,14 @@ __global__ __launch_bounds__(256) void window_pool_mfma_kernel(WindowMfmaParams 
       if (tail16) ktail[kb] = *reinterpret_cast<const bf16x4_t*>(knext[kb] + 32 * nk32 + 4 * lg);
     }
   };
-  if (AHEAD && ntiles > 0) {
-    prefetch(0);
+  // a split takes a contiguous share of the tiles
+  const int per_split = p.nsplit > 1 ? (ntiles + p.nsplit - 1) / p.nsplit : ntiles;
+  const int t_begin = split * per_split, t_end = min(ntiles, t_begin + per_split);
+  if (AHEAD && t_begin < t_end) {
+    prefetch(t_begin);
     if (active) fetch_k();
   }
-  for (int tile = 0; tile < ntiles; ++tile) {
+  for (int tile = t_begin; tile < t_end; ++tile) {
     const int phase = tile < npt ? 0 : 1;
     const int e0 = tile_start(tile);
     const int e_end = phase == 0 ? nbmax : i1 + 1;
@@ -201,7 +207,7 @@ __global__ __launch_bounds__(256) void window_pool_mfma_kernel(WindowMfmaParams 
       }
     }
     tile_barrier();
-    if (AHEAD && tile + 1 < ntiles) prefetch(tile + 1);
+    if (AHEAD && tile + 1 < t_end) prefetch(tile + 1);
     if (!active) continue;
     {
       float s[4][4];
@@ -226,7 +232,7 @@ __global__ __launch_bounds__(256) void window_pool_mfma_kernel(WindowMfmaParams 
           s[kb][i] = vis ? acc[i] * p.scale : -INFINITY;
         }
       }
-      if (AHEAD && tile + 1 < ntiles) fetch_k();                            // in flight across the softmax, PV and the barriers
+      if (AHEAD && tile + 1 < t_end) fetch_k();                            // in flight across the softmax, PV and the barriers
       float mx = -INFINITY;
 #pragma unroll
       for (int kb = 0; kb < 4; ++kb)
@@ -270,6 +276,18 @@ __global__ __launch_bounds__(256) void window_pool_mfma_kernel(WindowMfmaParams 
     }
   }
   if (!active || !qvalid) return;
+  if (p.nsplit > 1) {                                                       // unnormalised partials; window_pool_merge_kernel ends the job
+    float* w = p.ws + ((t * p.H + h) * p.nsplit + split) * (Dv + 4);
+#pragma unroll
+    for (int d = 0; d < kMaxDvb; ++d)
+      if (d < ndvb)
+        *reinterpret_cast<f32x4_t*>(w + 16 * d + 4 * lg) = acc_o[d];
+    if (lg == 0) {
+      w[Dv] = m;
+      w[Dv + 1] = l;
+    }
+    return;
+  }
   const float inv = l > 0.0f ? 1.0f / l : 0.0f;
   uint16_t* orow = p.out + (t * p.H + h) * Dv;
   const uint16_t* grow = p.gate != nullptr ? p.gate + t * p.ld_gate + static_cast<int64_t>(h) * Dv : nullptr;
@@ -287,6 +305,31 @@ __global__ __launch_bounds__(256) void window_pool_mfma_kernel(WindowMfmaParams 
   }
 }
 
+// One wave per (token, query head): combines the splits' partials (each with its own running maximum), applies the gate.
+__global__ __launch_bounds__(256) void window_pool_merge_kernel(const float* __restrict__ ws, const uint16_t* __restrict__ gate,
+                                                                int64_t ld_gate, uint16_t* __restrict__ out, int64_t items,
+                                                                int H, int Dv, int nsplit) {
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+  const int64_t item = static_cast<int64_t>(blockIdx.x) * (blockDim.x / kWave) + wave;
+  if (item >= items) return;
+  const int64_t t = item / H;
+  const int h = static_cast<int>(item - t * H);
+  const float* w = ws + item * nsplit * (Dv + 4);
+  float mm = 0.0f;
+  for (int s = 0; s < nsplit; ++s) mm = fmaxf(mm, w[s * (Dv + 4) + Dv]);
+  float ll = 0.0f;
+  for (int s = 0; s < nsplit; ++s) ll += w[s * (Dv + 4) + Dv + 1] * expf(w[s * (Dv + 4) + Dv] - mm);
+  const float inv = ll > 0.0f ? 1.0f / ll : 0.0f;
+  for (int dv = lane; dv < Dv; dv += kWave) {
+    float acc = 0.0f;
+    for (int s = 0; s < nsplit; ++s) acc += w[s * (Dv + 4) + dv] * expf(w[s * (Dv + 4) + Dv] - mm);
+    float val = acc * inv;
+    if (gate != nullptr)
+      val *= sigmoidf_(__builtin_bit_cast(float, static_cast<uint32_t>(gate[t * ld_gate + static_cast<int64_t>(h) * Dv + dv]) << 16));
+    out[item * Dv + dv] = static_cast<uint16_t>(bf16_bits(val));
+  }
+}
+
 }  // namespace lvmix
 
 using namespace lvmix;
@@ -295,7 +338,7 @@ extern "C" int lv_window_pool_attn_mfma(const void* q, const void* k_cache, cons
                                         const void* vp, const void* gate, int64_t ld_gate, void* out, const int32_t* cu_q,
                                         const int32_t* ctx_lens, const int32_t* block_tables, int bt_stride, int B,
                                         int max_new_tokens, int H, int G, int D, int Dv, int page, int window, int P,
-                                        float scale, int has_sink, void* stream) {
+                                        float scale, int has_sink, int nsplit, void* workspace, int64_t T, void* stream) {
   if (B == 0 || max_new_tokens <= 0) return 0;
   if (!q || !k_cache || !v_cache || !out || !cu_q || !ctx_lens || !block_tables)
     return fail(-1, "lv_window_pool_attn_mfma: null pointer");
@@ -311,9 +354,12 @@ extern "C" int lv_window_pool_attn_mfma(const void* q, const void* k_cache, cons
                      static_cast<const uint16_t*>(v_cache), static_cast<const uint16_t*>(kp),
                      static_cast<const uint16_t*>(vp), static_cast<const uint16_t*>(gate), ld_gate,
                      static_cast<uint16_t*>(out), cu_q, ctx_lens, block_tables, bt_stride, H, G, D, Dv, page, window, P,
-                     P > 0 ? (page + P - 1) / P : 0, ngroups, scale, has_sink ? 1.0f : 0.0f};
+                     P > 0 ? (page + P - 1) / P : 0, ngroups, scale, has_sink ? 1.0f : 0.0f,
+                     nsplit > 1 ? nsplit : 1, static_cast<float*>(workspace)};
+  if (nsplit > 1 && (max_new_tokens > kTileQ || workspace == nullptr || T <= 0))
+    return fail(-1, "lv_window_pool_attn_mfma: key splits need one query tile per sequence and a workspace");
   const size_t shm = static_cast<size_t>(Dv) * kLdk * sizeof(uint16_t);
-  dim3 grid((max_new_tokens + kTileQ - 1) / kTileQ, G * ngroups, B), block(256);
+  dim3 grid(nsplit > 1 ? nsplit : (max_new_tokens + kTileQ - 1) / kTileQ, G * ngroups, B), block(256);
   hipStream_t st = as_stream(stream);
   if (max_new_tokens <= kTileQ) {
     if (D <= 128) window_pool_mfma_kernel<true, 4><<<grid, block, shm, st>>>(p);
@@ -321,6 +367,12 @@ extern "C" int lv_window_pool_attn_mfma(const void* q, const void* k_cache, cons
   } else {
     if (D <= 128) window_pool_mfma_kernel<false, 4><<<grid, block, shm, st>>>(p);
     else window_pool_mfma_kernel<false, kMaxK32><<<grid, block, shm, st>>>(p);
+  }
+  if (nsplit > 1) {
+    const int64_t items = T * H;
+    window_pool_merge_kernel<<<dim3(static_cast<unsigned>((items + 3) / 4)), block, 0, st>>>(
+        static_cast<const float*>(workspace), static_cast<const uint16_t*>(gate), ld_gate, static_cast<uint16_t*>(out),
+        items, H, Dv, nsplit);
   }
   return launched("lv_window_pool_attn_mfma");
 }

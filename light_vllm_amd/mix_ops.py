@@ -280,12 +280,23 @@ def window_pool_attention(q, k_cache, v_cache, kp, vp, gate, step, H, G, D, Dv, 
         lib = _mixlib.load()
         if (WINDOW_ATTN_KERNEL == "auto" and q.dtype == torch.bfloat16 and D % 16 == 0 and Dv % 16 == 0
                 and D <= 256 and Dv <= 256):
+            # decode-shaped steps put one workgroup per (sequence, kv head) on the chip: cut each sequence's key
+            # tiles over enough workgroups to fill it (partials merged by a second kernel)
+            nsplit, ws = 1, None
+            B = len(step.host_lens_q)
+            if max(step.host_lens_q) <= 16:
+                most = max(c + n for c, n in zip(step.host_ctx_lens, step.host_lens_q))
+                tiles = -(-min(most, window + 16) // 64) + (-(-(max(most - window, 0) // P) // 64) if P > 0 else 0)
+                nsplit = max(1, min(tiles, 256 // max(B * G * -(-(H // G) // 4), 1), 32))
+                if nsplit > 1:
+                    ws = torch.empty(T * H * nsplit * (Dv + 4), dtype=torch.float32, device=q.device)
             _mixlib.check(lib.lv_window_pool_attn_mfma(_p(q), _p(k_cache), _p(v_cache), _p(kp), _p(vp), _p(gate),
                                                        gate.stride(0) if gate is not None else 0, _p(out), _p(step.cu_q),
                                                        _p(step.ctx_lens), _p(step.block_tables),
                                                        step.block_tables.stride(0), len(step.host_lens_q),
                                                        max(step.host_lens_q), H, G, D, Dv, page, window, P, scale,
-                                                       int(has_sink), _stream(q)), "lv_window_pool_attn_mfma")
+                                                       int(has_sink), nsplit, _p(ws), T, _stream(q)),
+                          "lv_window_pool_attn_mfma")
             return out
         _mixlib.check(lib.lv_window_pool_attn(_p(q), _p(k_cache), _p(v_cache), _p(kp), _p(vp), _p(gate),
                                               gate.stride(0) if gate is not None else 0, _p(out), _p(step.cu_q),

@@ -196,6 +196,14 @@ def case_window_pool_beacons(device, dtype):
         step = K.make_step([1] * len(rows), rows, [0] * len(rows), [table] * len(rows), device)
         got = mix_ops.window_pool_attention(qd[rows].contiguous(), kc, vc, kp, vp, None, step, H, G, D, Dv, window, P, scale, True)
         check(got, rows, "decode")
+        # few sequences: the matrix-core kernel then cuts each one's key tiles over several workgroups and merges
+        few = rows[-3:]
+        step = K.make_step([1] * len(few), few, [0] * len(few), [table] * len(few), device)
+        got = mix_ops.window_pool_attention(qd[few].contiguous(), kc, vc, kp, vp, None, step, H, G, D, Dv, window, P, scale, True)
+        check(got, few, "decode, few sequences")
+        step = K.make_step([2], [L - 2], [0], [table], device)
+        got = mix_ops.window_pool_attention(qd[L - 2:].contiguous(), kc, vc, kp, vp, None, step, H, G, D, Dv, window, P, scale, True)
+        check(got, [L - 2, L - 1], "two tokens behind a long context")
         a, b = L // 3, L // 3 + 2       # a portion of two tokens in the middle, beside one that starts a sequence
         step = K.make_step([b - a, 5], [a, 0], [0, 1], [table, table], device)
         got = mix_ops.window_pool_attention(torch.cat([qd[a:b], qd[:5]]).contiguous(), kc, vc, kp, vp, None, step,
