@@ -29,6 +29,7 @@ struct WindowMfmaParams {
   const int32_t *cu_q, *ctx_lens, *block_tables;
   int bt_stride, H, G, D, Dv, page, window, P, PP, ngroups;
   float scale, sink;
+  uint32_t m_page, m_P, m_nseg;   // floor(2^32 / d) of the three divisors the tile loop divides by (see fdiv)
   int nsplit;          // > 1 (launches of at most one query tile per sequence): grid.x = split of the key tiles
   float* ws;           // [T, H, nsplit, Dv + 4] partial read-outs, running maximum and sum
 };
@@ -40,16 +41,27 @@ constexpr int kLdk = kTileK + 4; // row stride (in keys) of the transposed V til
 constexpr int kMaxDvb = 16;    // Dv <= 256
 constexpr int kBtCache = 2048; // page ids of a sequence kept in LDS (longer sequences look them up in memory)
 
+// n / d for 0 <= n < 2^31 with magic = floor(2^32 / d) (0xffffffff for d = 1): the estimate is the quotient or one
+// less. The tile loop divides by the page size, the pool size and the row's segment count for every row address;
+// the compiler's general 32-bit division is some forty instructions each and dominated the kernel.
+__device__ __forceinline__ int fdiv(int n, int d, uint32_t magic) {
+  const uint32_t q = __umulhi(static_cast<uint32_t>(n), magic);
+  const uint32_t r = static_cast<uint32_t>(n) - q * static_cast<uint32_t>(d);
+  return static_cast<int>(r >= static_cast<uint32_t>(d) ? q + 1 : q);
+}
+
 __device__ __forceinline__ short bf16_bits(float x) {
   __bf16 b = static_cast<__bf16>(x);
   return __builtin_bit_cast(short, b);
 }
 
-// AHEAD: fetch the next tile's V rows, key-row addresses and (once the current scores are done) K fragments while
-// the current tile is computed. It pays when a launch has few workgroups per compute unit (single decoded tokens); a
-// prompt's many tiles hide latency by occupancy, which the extra registers would cost.
-template <bool AHEAD, int K32>
-__global__ __launch_bounds__(256) void window_pool_mfma_kernel(WindowMfmaParams p) {
+// AHEAD: the next tile's V rows, key-row addresses and (once the current scores are done) K fragments are fetched while
+// the current tile is computed. That pays when a launch has few workgroups per compute unit (decoded tokens). A prompt's
+// many tiles hide latency by occupancy instead, and every register counts there: with the 32 registers of a V tile held
+// ahead the kernel fell from two waves a SIMD to one and ran 1.7x slower; K32 and DVB size the fragment arrays for the
+// head sizes at hand for the same reason.
+template <bool AHEAD, int K32, int DVB>
+__global__ __launch_bounds__(256, (AHEAD || DVB > 8) ? 1 : 4) void window_pool_mfma_kernel(WindowMfmaParams p) {
   extern __shared__ uint16_t vs[];                      // V^T tile [Dv][kLdk]
   const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
   const int ln = lane & 15, lg = lane >> 4;
@@ -94,9 +106,9 @@ __global__ __launch_bounds__(256) void window_pool_mfma_kernel(WindowMfmaParams 
       if (kk < nk32) qf[kk] = *reinterpret_cast<const bf16x8_t*>(qrow + 32 * kk + 8 * lg);
     if (tail16) qtail = *reinterpret_cast<const bf16x4_t*>(qrow + 32 * nk32 + 4 * lg);
   }
-  f32x4_t acc_o[kMaxDvb];
+  f32x4_t acc_o[DVB];
 #pragma unroll
-  for (int d = 0; d < kMaxDvb; ++d) acc_o[d] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+  for (int d = 0; d < DVB; ++d) acc_o[d] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
   float m = 0.0f, l = split == 0 ? p.sink : 0.0f;
 
   const int nbmax = (P > 0 && i1 - W + 1 > 0) ? (i1 - W + 1) / P : 0;      // pooled blocks the last query sees
@@ -107,35 +119,40 @@ __global__ __launch_bounds__(256) void window_pool_mfma_kernel(WindowMfmaParams 
   const int npt = (nbmax + kTileK - 1) / kTileK;
   const int ntt = (i1 + 1 - jlo + kTileK - 1) / kTileK;
   const int ntiles = npt + ntt;
-  const int vrow_id = threadIdx.x >> 2, vq = threadIdx.x & 3;             // staging: 4 threads per V row
   const int nseg = Dv / 4;                                                // 8-byte segments of a row
 
   auto entry_rows = [&](int tile, int e, const uint16_t*& kr_, const uint16_t*& vr_) {
     if (tile < npt) {
       const int ec = min(e, nbmax - 1);
-      const int pj = (ec * P + P - 1) / page;
-      const int64_t slot = static_cast<int64_t>(bt(pj)) * p.PP + (ec - (page * pj) / P);
+      const int pj = fdiv(ec * P + P - 1, page, p.m_page);
+      const int64_t slot = static_cast<int64_t>(bt(pj)) * p.PP + (ec - fdiv(page * pj, P, p.m_P));
       kr_ = p.kp + slot * GD + g * D;
       vr_ = p.vp + slot * GDv + g * Dv;
     } else {
       const int ec = min(e, i1);
-      const int64_t slot = static_cast<int64_t>(bt(ec / page)) * page + ec % page;
+      const int pj = fdiv(ec, page, p.m_page);
+      const int64_t slot = static_cast<int64_t>(bt(pj)) * page + (ec - pj * page);
       kr_ = p.k_cache + slot * GD + g * D;
       vr_ = p.v_cache + slot * GDv + g * Dv;
     }
   };
   auto tile_start = [&](int tile) { return tile < npt ? tile * kTileK : jlo + (tile - npt) * kTileK; };
 
-  uint2 vreg[kMaxDvb];
+  // V rows of a tile: consecutive threads take consecutive 8-byte segments of a row (whole cache lines per load
+  // instruction). AHEAD: all of a thread's loads are issued together, one tile ahead of their use, and wait in registers.
+  uint2 vreg[AHEAD ? DVB : 1];
   const uint16_t* knext[4];
   auto prefetch = [&](int tile) {
     const int e0 = tile_start(tile);
-    const uint16_t *kr_, *vr_;
-    entry_rows(tile, e0 + vrow_id, kr_, vr_);
 #pragma unroll
-    for (int x = 0; x < kMaxDvb; ++x) {
-      const int seg = vq + 4 * x;
-      if (seg < nseg) vreg[x] = *reinterpret_cast<const uint2*>(vr_ + seg * 4);
+    for (int x = 0; x < (AHEAD ? DVB : 0); ++x) {
+      const int c = threadIdx.x + 256 * x;
+      if (c < kTileK * nseg) {
+        const int row = fdiv(c, nseg, p.m_nseg), seg = c - row * nseg;
+        const uint16_t *kr_, *vr_;
+        entry_rows(tile, e0 + row, kr_, vr_);
+        vreg[x] = *reinterpret_cast<const uint2*>(vr_ + seg * 4);
+      }
     }
 #pragma unroll
     for (int kb = 0; kb < 4; ++kb) {
@@ -143,17 +160,23 @@ __global__ __launch_bounds__(256) void window_pool_mfma_kernel(WindowMfmaParams 
       entry_rows(tile, e0 + kb * 16 + ln, knext[kb], unused);
     }
   };
-  // Only LDS traffic meets at the barriers of the tile loop. The fetch-ahead variant waits for that alone, so the
+  auto store_v = [&](uint16_t* dst, uint2 v4) {
+    dst[0] = static_cast<uint16_t>(v4.x & 0xffffu);
+    dst[kLdk] = static_cast<uint16_t>(v4.x >> 16);
+    dst[2 * kLdk] = static_cast<uint16_t>(v4.y & 0xffffu);
+    dst[3 * kLdk] = static_cast<uint16_t>(v4.y >> 16);
+  };
+  // Only LDS traffic meets at the barriers of the tile loop. The fetch-ahead variant waits for that alone, so that the
   // vector loads of the next tile stay in flight across them (a full __syncthreads would drain them every tile).
   auto tile_barrier = [&]() {
     if (AHEAD) asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
     else __syncthreads();
   };
-  bf16x8_t kdata[4][K32];
+  bf16x8_t kdata[AHEAD ? 4 : 1][K32];
   bf16x4_t ktail[4];
   auto fetch_k = [&]() {                                                    // the K fragments of the tile knext points to
 #pragma unroll
-    for (int kb = 0; kb < 4; ++kb) {
+    for (int kb = 0; kb < (AHEAD ? 4 : 0); ++kb) {
 #pragma unroll
       for (int kk = 0; kk < K32; ++kk)
         if (kk < nk32) kdata[kb][kk] = *reinterpret_cast<const bf16x8_t*>(knext[kb] + 32 * kk + 8 * lg);
@@ -173,32 +196,23 @@ __global__ __launch_bounds__(256) void window_pool_mfma_kernel(WindowMfmaParams 
     const int e_end = phase == 0 ? nbmax : i1 + 1;
     const uint16_t* kcur[4];
     tile_barrier();                                                         // the previous tile's V reads are done
-    if (AHEAD) {
+    if constexpr (AHEAD) {
 #pragma unroll
-      for (int x = 0; x < kMaxDvb; ++x) {
-        const int seg = vq + 4 * x;
-        if (seg < nseg) {
-          uint16_t* dst = vs + (seg * 4) * kLdk + vrow_id;
-          dst[0] = static_cast<uint16_t>(vreg[x].x & 0xffffu);
-          dst[kLdk] = static_cast<uint16_t>(vreg[x].x >> 16);
-          dst[2 * kLdk] = static_cast<uint16_t>(vreg[x].y & 0xffffu);
-          dst[3 * kLdk] = static_cast<uint16_t>(vreg[x].y >> 16);
+      for (int x = 0; x < DVB; ++x) {
+        const int c = threadIdx.x + 256 * x;
+        if (c < kTileK * nseg) {
+          const int row = fdiv(c, nseg, p.m_nseg), seg = c - row * nseg;
+          store_v(vs + (seg * 4) * kLdk + row, vreg[x]);
         }
       }
 #pragma unroll
       for (int kb = 0; kb < 4; ++kb) kcur[kb] = knext[kb];
     } else {
-      // consecutive threads take consecutive 8-byte segments of a row: whole cache lines per load instruction
       for (int c = threadIdx.x; c < kTileK * nseg; c += blockDim.x) {
-        const int row = c / nseg, seg = c - row * nseg;
+        const int row = fdiv(c, nseg, p.m_nseg), seg = c - row * nseg;
         const uint16_t *kr_, *vr_;
         entry_rows(tile, e0 + row, kr_, vr_);
-        const uint2 v4 = *reinterpret_cast<const uint2*>(vr_ + seg * 4);
-        uint16_t* dst = vs + (seg * 4) * kLdk + row;
-        dst[0] = static_cast<uint16_t>(v4.x & 0xffffu);
-        dst[kLdk] = static_cast<uint16_t>(v4.x >> 16);
-        dst[2 * kLdk] = static_cast<uint16_t>(v4.y & 0xffffu);
-        dst[3 * kLdk] = static_cast<uint16_t>(v4.y >> 16);
+        store_v(vs + (seg * 4) * kLdk + row, *reinterpret_cast<const uint2*>(vr_ + seg * 4));
       }
 #pragma unroll
       for (int kb = 0; kb < 4; ++kb) {
@@ -219,7 +233,7 @@ __global__ __launch_bounds__(256) void window_pool_mfma_kernel(WindowMfmaParams 
         for (int kk = 0; kk < K32; ++kk)
           if (kk < nk32)
             acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-                AHEAD ? kdata[kb][kk] : *reinterpret_cast<const bf16x8_t*>(krow + 32 * kk + 8 * lg), qf[kk], acc, 0, 0, 0);
+                AHEAD ? kdata[AHEAD ? kb : 0][kk] : *reinterpret_cast<const bf16x8_t*>(krow + 32 * kk + 8 * lg), qf[kk], acc, 0, 0, 0);
         if (tail16)
           acc = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(
               AHEAD ? ktail[kb] : *reinterpret_cast<const bf16x4_t*>(krow + 32 * nk32 + 4 * lg), qtail, acc, 0, 0, 0);
@@ -258,13 +272,13 @@ __global__ __launch_bounds__(256) void window_pool_mfma_kernel(WindowMfmaParams 
       l = l * corr + rs;
       m = nm;
 #pragma unroll
-      for (int d = 0; d < kMaxDvb; ++d)
+      for (int d = 0; d < DVB; ++d)
         if (d < ndvb) acc_o[d] *= corr;
 #pragma unroll
       for (int c = 0; c < 2; ++c) {
         const uint16_t* vt = vs + ln * kLdk + c * 32 + 4 * lg;              // value column ln: keys 4lg.. of blocks 2c, 2c+1
 #pragma unroll
-        for (int d = 0; d < kMaxDvb; ++d) {
+        for (int d = 0; d < DVB; ++d) {
           if (d < ndvb) {
             const uint2 lo = *reinterpret_cast<const uint2*>(vt + 16 * d * kLdk);
             const uint2 hi = *reinterpret_cast<const uint2*>(vt + 16 * d * kLdk + 16);
@@ -279,7 +293,7 @@ __global__ __launch_bounds__(256) void window_pool_mfma_kernel(WindowMfmaParams 
   if (p.nsplit > 1) {                                                       // unnormalised partials; window_pool_merge_kernel ends the job
     float* w = p.ws + ((t * p.H + h) * p.nsplit + split) * (Dv + 4);
 #pragma unroll
-    for (int d = 0; d < kMaxDvb; ++d)
+    for (int d = 0; d < DVB; ++d)
       if (d < ndvb)
         *reinterpret_cast<f32x4_t*>(w + 16 * d + 4 * lg) = acc_o[d];
     if (lg == 0) {
@@ -292,7 +306,7 @@ __global__ __launch_bounds__(256) void window_pool_mfma_kernel(WindowMfmaParams 
   uint16_t* orow = p.out + (t * p.H + h) * Dv;
   const uint16_t* grow = p.gate != nullptr ? p.gate + t * p.ld_gate + static_cast<int64_t>(h) * Dv : nullptr;
 #pragma unroll
-  for (int d = 0; d < kMaxDvb; ++d) {
+  for (int d = 0; d < DVB; ++d) {
     if (d < ndvb) {
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
@@ -334,6 +348,8 @@ __global__ __launch_bounds__(256) void window_pool_merge_kernel(const float* __r
 
 using namespace lvmix;
 
+static uint32_t magic(int d) { return d <= 1 ? 0xffffffffu : static_cast<uint32_t>((1ull << 32) / static_cast<uint64_t>(d)); }
+
 extern "C" int lv_window_pool_attn_mfma(const void* q, const void* k_cache, const void* v_cache, const void* kp,
                                         const void* vp, const void* gate, int64_t ld_gate, void* out, const int32_t* cu_q,
                                         const int32_t* ctx_lens, const int32_t* block_tables, int bt_stride, int B,
@@ -355,18 +371,19 @@ extern "C" int lv_window_pool_attn_mfma(const void* q, const void* k_cache, cons
                      static_cast<const uint16_t*>(vp), static_cast<const uint16_t*>(gate), ld_gate,
                      static_cast<uint16_t*>(out), cu_q, ctx_lens, block_tables, bt_stride, H, G, D, Dv, page, window, P,
                      P > 0 ? (page + P - 1) / P : 0, ngroups, scale, has_sink ? 1.0f : 0.0f,
-                     nsplit > 1 ? nsplit : 1, static_cast<float*>(workspace)};
+                     magic(page), magic(P > 0 ? P : 1), magic(Dv / 4), nsplit > 1 ? nsplit : 1, static_cast<float*>(workspace)};
   if (nsplit > 1 && (max_new_tokens > kTileQ || workspace == nullptr || T <= 0))
     return fail(-1, "lv_window_pool_attn_mfma: key splits need one query tile per sequence and a workspace");
   const size_t shm = static_cast<size_t>(Dv) * kLdk * sizeof(uint16_t);
   dim3 grid(nsplit > 1 ? nsplit : (max_new_tokens + kTileQ - 1) / kTileQ, G * ngroups, B), block(256);
   hipStream_t st = as_stream(stream);
+  const bool small = D <= 128 && Dv <= 128;
   if (max_new_tokens <= kTileQ) {
-    if (D <= 128) window_pool_mfma_kernel<true, 4><<<grid, block, shm, st>>>(p);
-    else window_pool_mfma_kernel<true, kMaxK32><<<grid, block, shm, st>>>(p);
+    if (small) window_pool_mfma_kernel<true, 4, 8><<<grid, block, shm, st>>>(p);
+    else window_pool_mfma_kernel<true, kMaxK32, kMaxDvb><<<grid, block, shm, st>>>(p);
   } else {
-    if (D <= 128) window_pool_mfma_kernel<false, 4><<<grid, block, shm, st>>>(p);
-    else window_pool_mfma_kernel<false, kMaxK32><<<grid, block, shm, st>>>(p);
+    if (small) window_pool_mfma_kernel<false, 4, 8><<<grid, block, shm, st>>>(p);
+    else window_pool_mfma_kernel<false, kMaxK32, kMaxDvb><<<grid, block, shm, st>>>(p);
   }
   if (nsplit > 1) {
     const int64_t items = T * H;
