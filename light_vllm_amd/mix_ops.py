@@ -287,7 +287,7 @@ def window_pool_attention(q, k_cache, v_cache, kp, vp, gate, step, H, G, D, Dv, 
             if max(step.host_lens_q) <= 16:
                 most = max(c + n for c, n in zip(step.host_ctx_lens, step.host_lens_q))
                 tiles = -(-min(most, window + 16) // 64) + (-(-(max(most - window, 0) // P) // 64) if P > 0 else 0)
-                nsplit = max(1, min(tiles, 256 // max(B * G * -(-(H // G) // 4), 1), 32))
+                nsplit = max(1, min(tiles, 256 // max(B * G * -(-(H // G) // 4), 1), 32))      # one workgroup a CU: more splits cost more in the merge than they gain (measured)
                 if nsplit > 1:
                     ws = torch.empty(T * H * nsplit * (Dv + 4), dtype=torch.float32, device=q.device)
             _mixlib.check(lib.lv_window_pool_attn_mfma(_p(q), _p(k_cache), _p(v_cache), _p(kp), _p(vp), _p(gate),
