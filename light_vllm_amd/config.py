@@ -6,7 +6,7 @@
 from __future__ import annotations
 
 import os
-from dataclasses import dataclass
+from dataclasses import dataclass, field
 from typing import Any, Optional
 
 
@@ -36,6 +36,7 @@ class Config:
     dtype: Optional[str] = None       # "bfloat16" | "float32": overrides the checkpoint's dtype (f32: models whose kernels have it)
     max_cache_tokens: int = -1        # ragged-step models: > 0 sizes the page pool for this many tokens instead of from free HBM
     long_prefill_token_threshold: int = 0   # ragged-step models: > 0 caps the prompt tokens one sequence gets per step
+    ragged: bool = field(default=False, init=False)   # set from the model class: it runs ragged steps (utils.context.RaggedStep)
 
     def __post_init__(self):
         assert 1 <= self.tensor_parallel_size <= 8

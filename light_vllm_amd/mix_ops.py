@@ -10,8 +10,6 @@ ctx_lens [B], slots [B], tok_seq [T], block_tables [B, n] and the same lengths a
 """
 from __future__ import annotations
 
-import math
-
 import torch
 import torch.nn.functional as F
 

@@ -149,7 +149,8 @@ def case_window_pool_beacons(device, dtype):
                                               (2, 2, 24, 4, 5, 21, 16, 120), (3, 3, 8, 8, 16, 0, 16, 90),
                                               # head sizes in multiples of 16: the matrix-core kernel in bf16
                                               (4, 2, 32, 16, 37, 5, 16, 300), (6, 2, 48, 32, 70, 12, 64, 410),
-                                              (9, 1, 64, 80, 130, 7, 32, 333), (2, 2, 16, 16, 3, 0, 16, 90)):
+                                              (9, 1, 64, 80, 130, 7, 32, 333), (2, 2, 16, 16, 3, 0, 16, 90),
+                                              (2, 1, 160, 144, 40, 9, 32, 200)):       # heads above 128: the wide instantiation
         g = torch.Generator().manual_seed(L)
         rep = H // G
         k = 0.05 * torch.randn(L, G, D, generator=g)
