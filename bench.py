@@ -603,7 +603,8 @@ def _engine_rates(hf_config, batch, prompt_len, new_tokens, **kw):
     prompts = [torch.randint(0, hf_config.vocab_size, (prompt_len,), generator=g).tolist() for _ in range(batch)]
     llm = LLM(None, hf_config=hf_config, max_num_seqs=batch, max_model_len=4096, max_num_batched_tokens=16384,
               random_seed=0, random_on_device=True, **kw)
-    llm.generate(prompts[:2], SamplingParams(temperature=0.0, max_tokens=2, ignore_eos=True))      # warm the libraries
+    warm = [torch.randint(0, hf_config.vocab_size, (prompt_len,), generator=g).tolist() for _ in range(batch)]
+    llm.generate(warm, SamplingParams(temperature=0.0, max_tokens=2, ignore_eos=True))   # other prompts, the timed shapes
     llm.generate(prompts, SamplingParams(temperature=0.0, max_tokens=new_tokens, ignore_eos=True))
     st = dict(llm.last_stats)
     llm.exit()
@@ -726,11 +727,16 @@ def mixers_leg(sizes, batch, prompt_len, new_tokens):
     for name in sizes:
         z = MIXER_SIZES[name]
         rec = {"size": name, **z}
+        cache_tokens = batch * 256 * (-(-(prompt_len + new_tokens) // 256))
         rec["kagalorn"] = _engine_rates(_kagalorn_config(z), batch, prompt_len, new_tokens, kvcache_block_size=256,
-                                        max_cache_tokens=batch * 256 * (-(-(prompt_len + new_tokens) // 256)))
+                                        max_cache_tokens=cache_tokens)
+        rec["kagalorn_graph"] = _engine_rates(_kagalorn_config(z), batch, prompt_len, new_tokens, kvcache_block_size=256,
+                                              max_cache_tokens=cache_tokens, enforce_eager=False)
         blocks = batch * (-(-(prompt_len + new_tokens) // 256)) + 8
         rec["qwen3_eager"] = _engine_rates(_qwen3_config(z), batch, prompt_len, new_tokens, num_kvcache_blocks=blocks,
                                            enforce_eager=True)
+        rec["qwen3_graph"] = _engine_rates(_qwen3_config(z), batch, prompt_len, new_tokens, num_kvcache_blocks=blocks,
+                                           enforce_eager=False)
         rec["kernels"] = _mixer_kernel_table(z, dev, batch, prompt_len)
         out["sizes"].append(rec)
     print(json.dumps(out), flush=True)

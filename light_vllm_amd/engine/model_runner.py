@@ -52,10 +52,11 @@ class ModelRunner:
         self.block_size = config.kvcache_block_size
         self.max_position = hf_config.max_position_embeddings
         Sequence.set_block_size(self.block_size)
-        # ragged-step models (recurrent / windowed mixers): one eager code path for prompts, portions and
-        # decoded tokens; their kernels come from liblvmix.so and the paged-attention library stays unloaded
+        # ragged-step models (recurrent / windowed mixers): one code path for prompts, portions and decoded tokens
+        # (steps of single tokens replay hipGraphs unless enforce_eager); their kernels come from liblvmix.so and the
+        # paged-attention library stays unloaded
         self.ragged = bool(getattr(config, "ragged", False))
-        self.enforce_eager = config.enforce_eager or self.ragged
+        self.enforce_eager = config.enforce_eager
         self.world_size = config.tensor_parallel_size
         self.rank = rank
         self.event = event
@@ -109,8 +110,10 @@ class ModelRunner:
                 self.warmup_model()
                 self.reserve_workspace()
                 self.allocate_kv_cache()
-            if not self.enforce_eager:
-                self.capture_graphs()
+            if not self.enforce_eager and self.on_gpu:
+                self.capture_ragged_graphs() if self.ragged else self.capture_graphs()
+            elif self.ragged:
+                self.enforce_eager = True
         finally:
             torch.set_default_device("cpu")
             torch.set_default_dtype(default_dtype)
@@ -305,8 +308,10 @@ class ModelRunner:
         assert num_blocks > 0, "not enough memory for the cache"
         cfg.num_kvcache_blocks = int(num_blocks)
         self.cache_sizing = dict(per_block=per_block, per_slot=per_slot, blocks=int(num_blocks), slots=num_slots)
+        # one page and one slot more than the managers hand out: where the padding rows of a replayed graph write
+        self.pad_page, self.pad_slot = int(num_blocks), num_slots
         for m in users:
-            m.bind_cache(int(num_blocks), self.block_size, num_slots, self.device, self.dtype)
+            m.bind_cache(int(num_blocks) + 1, self.block_size, num_slots + 1, self.device, self.dtype)
 
     # ------------------------------------------------------------------ step inputs
     def _check_positions(self, last_position: int) -> None:
@@ -456,6 +461,9 @@ class ModelRunner:
         """A scheduled ragged step: a token for every sequence whose known tokens end with this step,
         None for those that are still in the middle of their prompt."""
         done = [seq.num_computed_tokens + seq.num_scheduled_tokens == len(seq) for seq in seqs]
+        if (not self.enforce_eager and all(done) and all(seq.num_scheduled_tokens == 1 for seq in seqs)
+                and len(seqs) <= self.graph_bs[-1]):
+            return self._replay_decode(seqs, all_greedy)
         ends, at = [], 0
         for seq in seqs:
             at += seq.num_scheduled_tokens
@@ -471,6 +479,63 @@ class ModelRunner:
         reset_context()
         it = iter(tokens)
         return [next(it) if d else None for d in done]
+
+    @torch.inference_mode()
+    def capture_ragged_graphs(self):
+        """hipGraphs of the ragged forward pass for steps in which every sequence brings one token, per
+        batch-size bucket. What the kernels' launch geometry takes from a step's lengths on the host
+        (key-tile splits, pooled blocks completed) is fixed at its bound for a static step, so that one
+        capture serves every context length; padding rows write to a page and a state slot of their own."""
+        assert self.on_gpu and self.ragged
+        cfg, dev = self.config, self.device
+        self.graph_bs = self.decode_batch_buckets()
+        max_bs = self.graph_bs[-1]
+        width = -(-cfg.max_model_len // self.block_size)
+        i32 = dict(dtype=torch.int32, device=dev)
+        gv = dict(input_ids=torch.zeros(max_bs, dtype=torch.int64, device=dev),
+                  positions=torch.zeros(max_bs, dtype=torch.int64, device=dev),
+                  ctx_lens=torch.zeros(max_bs, **i32), slots=torch.full((max_bs,), self.pad_slot, **i32),
+                  block_tables=torch.full((max_bs, width), self.pad_page, **i32),
+                  cu_q=torch.arange(max_bs + 1, **i32), tok_seq=torch.arange(max_bs, **i32),
+                  outputs=torch.zeros(max_bs, cfg.hf_config.hidden_size, dtype=self.dtype, device=dev))
+        self.graphs, self.plan_graphs, self.graph_pool = {}, {}, None
+        for bs in reversed(self.graph_bs):
+            step = RaggedStep(gv["cu_q"][:bs + 1], gv["ctx_lens"][:bs], gv["slots"][:bs], gv["tok_seq"][:bs],
+                              gv["block_tables"][:bs], [1] * bs, [cfg.max_model_len - 1] * bs, [self.pad_slot] * bs,
+                              None, static=True)
+            set_context(False, ragged=step)
+            gv["outputs"][:bs] = self.model(gv["input_ids"][:bs], gv["positions"][:bs])     # warm run outside capture
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, pool=self.graph_pool):
+                gv["outputs"][:bs] = self.model(gv["input_ids"][:bs], gv["positions"][:bs])
+            if self.graph_pool is None:
+                self.graph_pool = graph.pool()
+            self.graphs[bs] = graph
+            torch.cuda.synchronize()
+            reset_context()
+        self.graph_vars = gv
+
+    def _replay_decode(self, seqs: list[Sequence], all_greedy: bool):
+        bs = len(seqs)
+        bucket = next(x for x in self.graph_bs if x >= bs)
+        gv = self.graph_vars
+        tables = self.prepare_block_tables(seqs)
+        for seq in seqs:
+            assert len(seq.block_table) * self.block_size >= seq.num_computed_tokens + 1 and seq.state_slot >= 0
+        gv["ctx_lens"][:bucket].zero_()
+        gv["slots"][:bucket].fill_(self.pad_slot)
+        gv["block_tables"][:bucket].fill_(self.pad_page)
+        gv["input_ids"][:bucket].zero_()
+        gv["input_ids"][:bs] = self._to_device([seq[seq.num_computed_tokens] for seq in seqs], torch.int64)
+        gv["ctx_lens"][:bs] = self._to_device([seq.num_computed_tokens for seq in seqs], torch.int32)
+        gv["slots"][:bs] = self._to_device([seq.state_slot for seq in seqs], torch.int32)
+        gv["block_tables"][:bs, :tables.size(1)] = tables
+        self.graphs[bucket].replay()
+        set_context(False)
+        logits = self.model.compute_logits(gv["outputs"][:bs])
+        tokens = self.sampler(logits, self.prepare_sample(seqs), all_greedy).tolist()
+        reset_context()
+        return tokens
 
     def prepare_sample(self, seqs: list[Sequence]) -> torch.Tensor:
         return self._to_device([seq.temperature for seq in seqs], torch.float32)

@@ -245,6 +245,8 @@ def pool_update(k_cache, v_cache, kp, vp, step, G, D, Dv, P):
     page = k_cache.size(1)
     new_blocks = [(c + n) // P - c // P for n, c in zip(step.host_lens_q, step.host_ctx_lens)]
     most = max(new_blocks, default=0)
+    if step.static:        # a replayed graph cannot know: always launch, the kernel leaves when no block was completed
+        most = max(-(-n // P) + 1 for n in step.host_lens_q)
     if most == 0:
         return
     if k_cache.is_cuda:

@@ -47,6 +47,7 @@ class RaggedStep:
     host_ctx_lens: list
     host_slots: list
     host_block_tables: list
+    static: bool = False          # captured into a hipGraph: launch geometry must not depend on this step's lengths
 
 
 _CONTEXT = Context()

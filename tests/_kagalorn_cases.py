@@ -313,7 +313,7 @@ def case_engine_long_decode(device, dtype, tmp_path):
     K.assert_close(got["a"], want["a"], dtype, "long decode")
 
 
-def case_generate(device, tmp_path):
+def case_generate(device, tmp_path, enforce_eager=True):
     """Greedy generation through LLM.generate: the scheduler admits, cuts prompts into portions under a small
     token budget, mixes them with decoding sequences, preempts nothing it need not, and every completion is
     the oracle's greedy continuation."""
@@ -324,7 +324,8 @@ def case_generate(device, tmp_path):
     prompts = [K.tokens_for(cfg, n, 30 + n) for n in (19, 5, 33, 12, 8)]
     steps = 6
     llm = LLM(model_dir, dtype="float32", device=device, kvcache_block_size=16, max_num_seqs=3, max_cache_tokens=160,
-              max_num_batched_tokens=24, long_prefill_token_threshold=10, max_model_len=64)
+              max_num_batched_tokens=24, long_prefill_token_threshold=10, max_model_len=64, enforce_eager=enforce_eager)
+    assert llm.model_runner.enforce_eager == enforce_eager
     outs = llm.generate([list(p) for p in prompts], SamplingParams(temperature=0.0, max_tokens=steps, ignore_eos=True))
     llm.exit()
     for p, out in zip(prompts, outs):

@@ -69,3 +69,9 @@ def test_generate_greedy(gpu, tmp_path):
 
 def test_generate_under_preemption(gpu, tmp_path):
     C.case_generate_preemption(DEV, tmp_path)
+
+
+def test_generate_greedy_from_graphs(gpu, tmp_path):
+    """Steps of single tokens replay captured hipGraphs (buckets of 1, 2 and 4 sequences here, padded rows
+    included, many replays between eager prompt steps): the completions are the oracle's all the same."""
+    C.case_generate(DEV, tmp_path, enforce_eager=False)
