@@ -671,11 +671,12 @@ def _mixer_kernel_table(z, dev, batch, prompt_len):
         conv_state = torch.zeros(batch, 3, C, device=dev, dtype=bf)
         A_log, dt_bias = torch.zeros(H, device=dev), torch.zeros(H, device=dev)
         state = torch.zeros(batch, H, D, D, device=dev)
+        a_in = proj[:, C + H * D + H:C + H * D + 2 * H]
         add("delta_prep", phase, lambda: mix_ops.delta_prep(proj, conv_w, conv_state, A_log, dt_bias, step, G, H, D, D, 4,
-                                                            C + H * D, C + H * D + H, 1e-6),
+                                                            C + H * D, a_in, 1e-6),
             nbytes=T * (C * 2 + C * 4 + 8 * H))
         qn, kn, v, beta, dec = mix_ops.delta_prep(proj, conv_w, conv_state, A_log, dt_bias, step, G, H, D, D, 4,
-                                                  C + H * D, C + H * D + H, 1e-6)
+                                                  C + H * D, a_in, 1e-6)
         st_bytes = batch * H * D * D * 4 * 2
         add("gated_delta_rule", phase, lambda: mix_ops.gated_delta_rule(qn, kn, v, beta, dec, state, step),
             nbytes=st_bytes + T * (2 * G * D + 2 * H * D) * 4, flops=T * H * D * D * 2 * 3)

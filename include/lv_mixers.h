@@ -4,6 +4,7 @@
  *
  *   lv_hc_update_norm        hyper-connection stream update fused with the next sublayer's stream
  *                            read-out and grouped RMS norm
+ *   lv_residual_add_norm     single f32 residual: adds up to two sublayer outputs, RMS norm with weight (offset + w)
  *   lv_clamped_glu           clamped gated linear unit  min(g, L) * sigmoid(alpha g) * (clamp(u, -L, L) + 1)
  *   lv_delta_prep            short causal convolution + silu over the q/k/v channels of a ragged step,
  *                            unit-norm q and k, write strength and decay of the gated delta rule
@@ -13,7 +14,15 @@
  *   lv_qk_fullnorm_store     RMS norm over the whole q and k projection, K/V scatter into the paged cache
  *   lv_pool_update           means of completed blocks of P cached keys and values
  *   lv_window_pool_attn      sliding-window attention over cached tokens plus pooled blocks that lie
- *                            before the window, softmax with a zero-score sink, sigmoid output gate
+ *                            before the window, softmax with an optional zero-score sink, sigmoid output gate;
+ *                            with a window no sequence reaches, no pool and no sink it is plain causal attention,
+ *                            and with row strides of their own K and V may be views of one wider cache row
+ *   lv_latent_prep           latent attention: RMS norm of the query latent, RMS norm of the key/value latent and
+ *                            rotation of the shared positional key part, both written into the paged latent cache
+ *   lv_latent_q_finish       joins the absorbed queries with their rotated positional part
+ *   lv_latent_out_gate       per-head outputs [H, T, Dv] -> [T, H*Dv] times sigmoid(gate), gate per head or per channel
+ *   lv_moe_route             sigmoid router with a selection-only correction, group limit and top-k
+ *   lv_relu2_scale           squared relu of the experts' up projections times the routing weight
  *
  * A "ragged step" is a batch of B sequences; sequence b brings cu_q[b+1]-cu_q[b] new tokens that
  * follow ctx_lens[b] tokens already in the cache / state (a whole prompt, a portion of one, or one
@@ -35,10 +44,14 @@
 extern "C" {
 #endif
 
-#define LV_MIX_ABI_VERSION 4
+#define LV_MIX_ABI_VERSION 5
 #define LV_MIX_BF16 0
 #define LV_MIX_F32 1
 #define LV_MIX_MAX_STREAMS 8
+#define LV_MIX_GATE_SILU 0
+#define LV_MIX_GATE_SIGMOID 1
+#define LV_MIX_GATE_PER_HEAD 0
+#define LV_MIX_GATE_PER_CHANNEL 1
 
 int lv_mix_abi_version(void);
 const char* lv_mix_last_error(void);
@@ -50,32 +63,41 @@ int lv_hc_update_norm(void* x, const void* y, const void* mix, const void* out_w
                       const void* norm_w, void* out, int64_t T, int S, int W, int groups, float eps,
                       int dtype, void* stream);
 
+/* x f32 [T, W] += y1 + y2 (act [T, W], either may be NULL), in place; when out != NULL:
+ * out act [T, W] = x / sqrt(mean(x^2) + eps) * (w_offset + w), w f32 [W]. */
+int lv_residual_add_norm(void* x, const void* y1, const void* y2, const void* w, float w_offset, void* out, int64_t T,
+                         int W, float eps, int dtype, void* stream);
+
 /* in act [T, 2F] (row stride ld_in) = [gate | up];  out act [T, F]. */
 int lv_clamped_glu(const void* in, int64_t ld_in, void* out, int64_t T, int F, float limit, float alpha,
                    int dtype, void* stream);
 
 /* proj act [T, ld]: columns [0, G*D) q, [G*D, 2*G*D) k, [2*G*D, 2*G*D + H*Dv) v (the convolution
- * channels, C of them), b at column off_b (H wide), a at column off_a (H wide).
+ * channels, C of them), b at column off_b (H wide). a act, rows of stride ld_a: the decay inputs, H numbers, or with
+ * decay_per_channel H*D (one for each key channel of each head; dt_bias is as wide as a row of a, A_log always [H]).
  * conv_w f32 [C, taps] (last column = current token); conv_state act [slots, taps-1, C].
- * Outputs f32: qn [T, G, D] (unit norm times D^-1/2), kn [T, G, D], v [T, H, Dv], beta [T, H], decay [T, H]. */
+ * Outputs f32: qn [T, G, D] (unit norm times D^-1/2), kn [T, G, D], v [T, H, Dv], beta [T, H],
+ * decay [T, H] or [T, H, D] = exp(-exp(A_log) * softplus(a + dt_bias)). */
 int lv_delta_prep(const void* proj, int64_t ld, const void* conv_w, const void* conv_state,
                   const void* A_log, const void* dt_bias, const int32_t* cu_q, const int32_t* ctx_lens,
                   const int32_t* slots, const int32_t* tok_seq, void* qn, void* kn, void* v, void* beta,
-                  void* decay, int64_t T, int G, int H, int D, int Dv, int taps, int off_b, int off_a,
-                  float unit_eps, int dtype, void* stream);
+                  void* decay, int64_t T, int G, int H, int D, int Dv, int taps, int off_b, const void* a,
+                  int64_t ld_a, int decay_per_channel, float unit_eps, int dtype, void* stream);
 
 int lv_conv_state_update(const void* proj, int64_t ld, void* conv_state, const int32_t* cu_q,
                          const int32_t* ctx_lens, const int32_t* slots, int B, int C, int taps, int dtype,
                          void* stream);
 
-/* state f32 [slots, H, D, Dv], read unless ctx_lens[b] == 0, written back.  o f32 [T, H, Dv]. */
+/* state f32 [slots, H, D, Dv], read unless ctx_lens[b] == 0, written back.  o f32 [T, H, Dv].
+ * decay f32 [T, H], or [T, H, D] with decay_per_channel: row d of a head's state is multiplied by its own number. */
 int lv_gated_delta_rule(const void* qn, const void* kn, const void* v, const void* beta, const void* decay,
                         void* state, const int32_t* cu_q, const int32_t* ctx_lens, const int32_t* slots,
-                        void* o, int B, int G, int H, int D, int Dv, void* stream);
+                        void* o, int B, int G, int H, int D, int Dv, int decay_per_channel, void* stream);
 
-/* out act [T, H*Dv] = o / sqrt(mean_dv(o^2) + eps) * norm_w[dv] * silu(gate);  gate act rows of stride ld_gate. */
+/* out act [T, H*Dv] = o / sqrt(mean_dv(o^2) + eps) * norm_w[dv] * act(gate), act = silu or sigmoid (LV_MIX_GATE_*);
+ * gate act rows of stride ld_gate. */
 int lv_head_norm_gate(const void* o, const void* gate, int64_t ld_gate, const void* norm_w, void* out,
-                      int64_t T, int H, int Dv, float eps, int dtype, void* stream);
+                      int64_t T, int H, int Dv, float eps, int gate_act, int dtype, void* stream);
 
 /* q act [T, H*D] (row stride ld), k [T, G*D], v [T, G*Dv] rows of the same stride.  q_out act [T, H*D]
  * contiguous = rms_norm(q over all H*D) * q_w; k likewise into k_cache [pages, page, G, D]; v copied into
@@ -96,12 +118,13 @@ int lv_pool_update(const void* k_cache, const void* v_cache, void* kp, void* vp,
 /* Query at position i sees cached positions j with 0 <= i-j < window and every pooled block b with
  * b*P + P - 1 <= i - window (P == 0: no pooled blocks); weights exp(s) / (sink + sum exp(s)) with
  * sink = 1 for has_sink, else 0.  gate (optional) act rows of stride ld_gate: out *= sigmoid(gate).
- * q act [T, H*D] contiguous; out act [T, H*Dv]. */
+ * q act [T, H*D] contiguous; out act [T, H*Dv].  k_ld, v_ld: elements between two tokens' rows in k_cache and v_cache
+ * (0: G*D and G*Dv); the pooled caches are always dense. */
 int lv_window_pool_attn(const void* q, const void* k_cache, const void* v_cache, const void* kp, const void* vp,
                         const void* gate, int64_t ld_gate, void* out, const int32_t* cu_q, const int32_t* ctx_lens,
                         const int32_t* tok_seq, const int32_t* block_tables, int bt_stride, int64_t T, int H, int G,
-                        int D, int Dv, int page, int window, int P, float scale, int has_sink, int dtype,
-                        void* stream);
+                        int D, int Dv, int page, int window, int P, float scale, int has_sink, int64_t k_ld,
+                        int64_t v_ld, int dtype, void* stream);
 
 /* The same attention on the matrix cores: bf16 only, D and Dv multiples of 16 up to 256. Tiles of 16 new
  * tokens per sequence; max_new_tokens = the largest cu_q[b+1] - cu_q[b] of the step.
@@ -111,7 +134,40 @@ int lv_window_pool_attn_mfma(const void* q, const void* k_cache, const void* v_c
                              const void* gate, int64_t ld_gate, void* out, const int32_t* cu_q, const int32_t* ctx_lens,
                              const int32_t* block_tables, int bt_stride, int B, int max_new_tokens, int H, int G, int D,
                              int Dv, int page, int window, int P, float scale, int has_sink, int nsplit, void* workspace,
-                             int64_t T, void* stream);
+                             int64_t T, int64_t k_ld, int64_t v_ld, void* stream);
+
+/* Latent attention, step 1. proj act [T, ld]: the query latent at column off_q (Rq wide), the key/value latent at
+ * off_kv (R wide) directly followed by the positional key part (Dr wide, may be 0).
+ * cq_out act [T, Rq] = rms_norm(query latent) * q_w.  cache act [pages, page, R + Dr]: the row of each token's position
+ * receives rms_norm(latent) * kv_w | rotated positional part.  Rotation: of the first rot_dims (even, <= Dr) entries,
+ * entry i pairs with i + rot_dims/2, angle = position * inv_freq[i] (inv_freq f32 [rot_dims/2]). */
+int lv_latent_prep(const void* proj, int64_t ld, int off_q, int off_kv, const void* q_w, const void* kv_w,
+                   const void* inv_freq, void* cq_out, void* cache, const int32_t* cu_q, const int32_t* ctx_lens,
+                   const int32_t* tok_seq, const int32_t* block_tables, int bt_stride, int64_t T, int Rq, int R, int Dr,
+                   int rot_dims, int page, float eps, int dtype, void* stream);
+
+/* Latent attention, step 2. q act [T, H, Dn + Dr] (the rotated part last), q_lat act [H, T, R] (the unrotated part
+ * already multiplied into the latent space).  q_out act [T, H, R + Dr] = q_lat | rotate(q[.., Dn:], position). */
+int lv_latent_q_finish(const void* q, const void* q_lat, const void* inv_freq, void* q_out, const int32_t* cu_q,
+                       const int32_t* ctx_lens, const int32_t* tok_seq, int64_t T, int H, int Dn, int Dr, int R,
+                       int rot_dims, int dtype, void* stream);
+
+/* o act [H, T, Dv] -> out act [T, H*Dv] = o * sigmoid(gate); gate act rows of stride ld_gate holding H numbers
+ * (LV_MIX_GATE_PER_HEAD) or H*Dv (LV_MIX_GATE_PER_CHANNEL). */
+int lv_latent_out_gate(const void* o, const void* gate, int64_t ld_gate, int gate_kind, void* out, int64_t T, int H,
+                       int Dv, int dtype, void* stream);
+
+/* Router of a mixture of experts. logits f32 [T, E]; scores s = sigmoid(logits); selection scores c = s + correction
+ * (f32 [E], may be NULL). The experts are split into `groups` consecutive blocks of equal size; a block is ranked by its
+ * two highest selection scores added up (by its one, for blocks of one expert); experts outside the `keep` highest-ranked blocks are excluded
+ * (groups <= 1: all). The `top` largest c are chosen (ties: lowest index first); weights = their s / (sum + 1e-20).
+ * ids int32 [T, top], weights f32 [T, top], dense f32 [T, E] (weights at the chosen experts, 0 elsewhere; may be NULL). */
+int lv_moe_route(const void* logits, const void* correction, void* ids, void* weights, void* dense, int64_t T, int E,
+                 int top, int groups, int keep, void* stream);
+
+/* up act [T, E*F] (all experts' up projections side by side), dense f32 [T, E]:
+ * out act [T, E*F] = relu(up)^2 * dense[t, e]. */
+int lv_relu2_scale(const void* up, const void* dense, void* out, int64_t T, int E, int F, int dtype, void* stream);
 
 #ifdef __cplusplus
 }

@@ -1,5 +1,6 @@
 """ctypes binding of liblvmix.so (include/lv_mixers.h): the kernels of the recurrent and windowed
-sequence mixers, the hyper-connection residual streams and the clamped gated unit.
+sequence mixers (delta rule, windowed and latent attention), the residual streams, the gated units
+and the mixture-of-experts router.
 
 The library is separate from liblvattn.so so that a model that needs only these kernels builds
 only these: `load()` compiles the sources once when no built library is there (a fresh checkout),
@@ -15,28 +16,36 @@ from ctypes import c_char_p, c_float, c_int, c_int64, c_void_p
 _HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(_HERE, "csrc", "mixers")
 LIB_PATH = os.path.join(_HERE, "lib", "liblvmix.so")
-SOURCES = ["mix_stream.hip", "mix_window_attn.hip", "mix_window_mfma.hip"]
-ABI_VERSION = 4
+SOURCES = ["mix_stream.hip", "mix_window_attn.hip", "mix_window_mfma.hip", "mix_latent.hip"]
+ABI_VERSION = 5
 
 _P = c_void_p
 SIGNATURES = {
     "lv_mix_abi_version": (c_int, []),
     "lv_mix_last_error": (c_char_p, []),
     "lv_hc_update_norm": (c_int, [_P, _P, _P, _P, _P, _P, _P, c_int64, c_int, c_int, c_int, c_float, c_int, _P]),
+    "lv_residual_add_norm": (c_int, [_P, _P, _P, _P, c_float, _P, c_int64, c_int, c_float, c_int, _P]),
     "lv_clamped_glu": (c_int, [_P, c_int64, _P, c_int64, c_int, c_float, c_float, c_int, _P]),
     "lv_delta_prep": (c_int, [_P, c_int64, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, c_int64,
-                              c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, _P]),
+                              c_int, c_int, c_int, c_int, c_int, c_int, _P, c_int64, c_int, c_float, c_int, _P]),
     "lv_conv_state_update": (c_int, [_P, c_int64, _P, _P, _P, _P, c_int, c_int, c_int, c_int, _P]),
-    "lv_gated_delta_rule": (c_int, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, _P]),
-    "lv_head_norm_gate": (c_int, [_P, _P, c_int64, _P, _P, c_int64, c_int, c_int, c_float, c_int, _P]),
+    "lv_gated_delta_rule": (c_int, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_int, _P]),
+    "lv_head_norm_gate": (c_int, [_P, _P, c_int64, _P, _P, c_int64, c_int, c_int, c_float, c_int, c_int, _P]),
     "lv_qk_fullnorm_store": (c_int, [_P, _P, _P, c_int64, _P, _P, _P, _P, _P, _P, _P, _P, _P, c_int, c_int64,
                                      c_int, c_int, c_int, c_int, c_int, c_float, c_int, _P]),
     "lv_pool_update": (c_int, [_P, _P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
                                c_int, c_int, _P]),
     "lv_window_pool_attn": (c_int, [_P, _P, _P, _P, _P, _P, c_int64, _P, _P, _P, _P, _P, c_int, c_int64, c_int,
-                                    c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, _P]),
+                                    c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int64, c_int64, c_int, _P]),
     "lv_window_pool_attn_mfma": (c_int, [_P, _P, _P, _P, _P, _P, c_int64, _P, _P, _P, _P, c_int, c_int, c_int, c_int,
-                                         c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, _P, c_int64, _P]),
+                                         c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, _P, c_int64,
+                                         c_int64, c_int64, _P]),
+    "lv_latent_prep": (c_int, [_P, c_int64, c_int, c_int, _P, _P, _P, _P, _P, _P, _P, _P, _P, c_int, c_int64, c_int, c_int,
+                               c_int, c_int, c_int, c_float, c_int, _P]),
+    "lv_latent_q_finish": (c_int, [_P, _P, _P, _P, _P, _P, _P, c_int64, c_int, c_int, c_int, c_int, c_int, c_int, _P]),
+    "lv_latent_out_gate": (c_int, [_P, _P, c_int64, c_int, _P, c_int64, c_int, c_int, c_int, _P]),
+    "lv_moe_route": (c_int, [_P, _P, _P, _P, _P, c_int64, c_int, c_int, c_int, c_int, _P]),
+    "lv_relu2_scale": (c_int, [_P, _P, _P, c_int64, c_int, c_int, c_int, _P]),
 }
 
 _lib = None

@@ -3,14 +3,18 @@
 //   hc_update_norm_kernel     one workgroup per token: the S residual streams are remixed and receive the
 //                             sublayer output, and in the same pass the next sublayer's input is read out
 //                             of them and normalised in groups. Streams and all arithmetic are f32.
+//   residual_add_norm_kernel  one workgroup per token: the single f32 residual receives the sum of up to two
+//                             sublayer outputs and is normalised for the next layer, weight (offset + w).
 //   clamped_glu_kernel        elementwise gate of the feed-forward.
 //   delta_prep_kernel         one wave per (token, head slot): convolution taps from the step's own rows
 //                             or the carried state, silu, unit norm; one more wave per token for the
-//                             write strength and the decay.
+//                             write strength and the decay (one per head, or one wave per head when every
+//                             key channel has a decay of its own).
 //   conv_state_update_kernel  one thread per (sequence, channel) shifts the carried inputs.
 //   gated_delta_rule_kernel   one workgroup per (64 value columns, head, sequence) walks the step's tokens;
 //                             each lane owns one column of the state, the four waves own a quarter of the
-//                             rows each, partial dot products meet in LDS once per token.
+//                             rows each, partial dot products meet in LDS once per token. The decay is one
+//                             number per head, or one for each key channel of it (a row of the state).
 //   head_norm_gate_kernel     one wave per (token, head).
 #include "mix_common.h"
 
@@ -120,6 +124,36 @@ static int hc_launch(void* x, const void* y, const void* mix, const void* out_w,
 }
 
 // ------------------------------------------------------------------------------------------------
+// x f32 [T, W] += y1 + y2 (either may be absent); out = x / sqrt(mean(x^2) + eps) * (w_offset + w).
+template <typename T>
+__global__ __launch_bounds__(256) void residual_add_norm_kernel(float* __restrict__ x, const T* __restrict__ y1,
+                                                                 const T* __restrict__ y2, const float* __restrict__ w,
+                                                                 float w_offset, T* __restrict__ out, int W, float eps) {
+  extern __shared__ float lds[];          // [W] the updated row, then [4] partial sums
+  float* red = lds + W;
+  const int64_t t = blockIdx.x;
+  float* xt = x + t * W;
+  float ss = 0.0f;
+  for (int i = threadIdx.x; i < W; i += blockDim.x) {
+    float v = xt[i];
+    if (y1 != nullptr || y2 != nullptr) {
+      float add = y1 != nullptr ? ldf(y1 + t * W + i) : 0.0f;
+      if (y2 != nullptr) add += ldf(y2 + t * W + i);
+      v += add;
+      xt[i] = v;
+    }
+    lds[i] = v;
+    ss += v * v;
+  }
+  if (out == nullptr) return;
+  ss = wave_sum(ss);
+  if (threadIdx.x % kWave == 0) red[threadIdx.x / kWave] = ss;
+  __syncthreads();
+  const float inv = 1.0f / sqrtf((red[0] + red[1] + red[2] + red[3]) / static_cast<float>(W) + eps);
+  for (int i = threadIdx.x; i < W; i += blockDim.x) stf(out + t * W + i, lds[i] * inv * (w_offset + w[i]));
+}
+
+// ------------------------------------------------------------------------------------------------
 template <typename T>
 __global__ __launch_bounds__(256) void clamped_glu_kernel(const T* __restrict__ in, int64_t ld_in, T* __restrict__ out,
                                                           int64_t Tn, int F, float limit, float alpha) {
@@ -174,8 +208,11 @@ struct DeltaPrepParams {
   const int32_t *cu_q, *ctx_lens, *slots, *tok_seq;
   float *qn, *kn, *v, *beta, *decay;
   int64_t T;
-  int G, H, D, Dv, taps, off_b, off_a;
+  int G, H, D, Dv, taps, off_b;
   float unit_eps;
+  const void* a;      // decay inputs, rows of stride ld_a: H numbers, or H * D when dec_dim == D
+  int64_t ld_a;
+  int dec_dim;        // 1: one decay per head; D: one for each of its key channels (dt_bias is as wide as a row of a)
 };
 
 template <typename T>
@@ -183,19 +220,29 @@ __global__ __launch_bounds__(256) void delta_prep_kernel(DeltaPrepParams p) {
   const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
   const int64_t t = blockIdx.x;
   const int unit = blockIdx.y * (blockDim.x / kWave) + wave;
-  const int units = 2 * p.G + p.H + 1;
+  const int base_units = 2 * p.G + p.H + 1;
+  const int units = base_units + (p.dec_dim > 1 ? p.H : 0);
   if (unit >= units) return;
   const T* proj = static_cast<const T*>(p.proj);
+  const T* arow = static_cast<const T*>(p.a) + blockIdx.x * p.ld_a;
+  if (unit >= base_units) {                       // decays of one head, one per key channel
+    const int h = unit - base_units;
+    const float rate = expf(p.A_log[h]);
+    for (int d = lane; d < p.dec_dim; d += kWave) {
+      const int i = h * p.dec_dim + d;
+      p.decay[blockIdx.x * static_cast<int64_t>(p.H) * p.dec_dim + i] = expf(-rate * softplusf_(ldf(arow + i) + p.dt_bias[i]));
+    }
+    return;
+  }
   const int b = p.tok_seq[t];
   const int q0 = p.cu_q[b];
   const int r = static_cast<int>(t) - q0;         // index of the token inside its sequence's portion
   const int ctx = p.ctx_lens[b];
-  if (unit == units - 1) {                        // write strength and decay, one lane per head
+  if (unit == base_units - 1) {                   // write strength and (per-head) decay, one lane per head
     for (int h = lane; h < p.H; h += kWave) {
       const float bv = ldf(proj + t * p.ld + p.off_b + h);
-      const float av = ldf(proj + t * p.ld + p.off_a + h);
       p.beta[t * p.H + h] = sigmoidf_(bv);
-      p.decay[t * p.H + h] = expf(-expf(p.A_log[h]) * softplusf_(av + p.dt_bias[h]));
+      if (p.dec_dim == 1) p.decay[t * p.H + h] = expf(-expf(p.A_log[h]) * softplusf_(ldf(arow + h) + p.dt_bias[h]));
     }
     return;
   }
@@ -265,6 +312,7 @@ struct DeltaRuleParams {
   float* o;
   int G, H, D, Dv;
 };
+// decay: [T, H] (one number per head) or, in the kernel's CH form, [T, H, D] (one per row of the state).
 
 // DR = rows of the state each of the four waves owns (4 * DR >= D; rows beyond D stay zero).
 // Tokens are taken in chunks of kDeltaChunk: the chunk's unit keys and queries, values, write strengths and
@@ -272,7 +320,7 @@ struct DeltaRuleParams {
 // per token), then each token costs LDS reads, 2 * DR multiply-adds per lane and one barrier.
 constexpr int kDeltaChunk = 16;
 
-template <int DR>
+template <int DR, bool CH>
 __global__ __launch_bounds__(256) void gated_delta_rule_kernel(DeltaRuleParams p) {
   extern __shared__ __attribute__((aligned(16))) float dl[];
   constexpr int DP = 4 * DR;                       // padded key size
@@ -283,6 +331,7 @@ __global__ __launch_bounds__(256) void gated_delta_rule_kernel(DeltaRuleParams p
   float* part_k = bd_lds + kDeltaChunk * 2;        // [2][4][64]
   float* part_o = part_k + 2 * 4 * kWave;          // [2][4][64]
   float* o_lds = part_o + 2 * 4 * kWave;           // [chunk][64]: read-outs leave for memory once per chunk
+  float* g_lds = o_lds + kDeltaChunk * kWave;      // CH: [chunk][DP] decays per row
   const int lane = threadIdx.x % kWave, rp = threadIdx.x / kWave;
   const int col = blockIdx.x * kWave + lane;
   const int h = blockIdx.y, b = blockIdx.z;
@@ -307,6 +356,7 @@ __global__ __launch_bounds__(256) void gated_delta_rule_kernel(DeltaRuleParams p
       const bool in = d < p.D;
       k_lds[x] = in ? p.kn[(t * p.G + g) * p.D + d] : 0.0f;
       q_lds[x] = in ? p.qn[(t * p.G + g) * p.D + d] : 0.0f;
+      if (CH) g_lds[x] = in ? p.decay[(t * p.H + h) * p.D + d] : 1.0f;
     }
     for (int x = threadIdx.x; x < cn * kWave; x += blockDim.x) {
       const int tok = x / kWave, cc = blockIdx.x * kWave + (x % kWave);
@@ -316,7 +366,7 @@ __global__ __launch_bounds__(256) void gated_delta_rule_kernel(DeltaRuleParams p
     if (threadIdx.x < cn) {
       const int64_t t = q0 + c0 + threadIdx.x;
       bd_lds[threadIdx.x * 2] = p.beta[t * p.H + h];
-      bd_lds[threadIdx.x * 2 + 1] = p.decay[t * p.H + h];
+      bd_lds[threadIdx.x * 2 + 1] = CH ? 1.0f : p.decay[t * p.H + h];
     }
     __syncthreads();
     for (int i = 0; i < cn; ++i) {
@@ -328,6 +378,13 @@ __global__ __launch_bounds__(256) void gated_delta_rule_kernel(DeltaRuleParams p
         const float4 q4 = *reinterpret_cast<const float4*>(q_lds + i * DP + row0 + r);
         kr[r] = k4.x; kr[r + 1] = k4.y; kr[r + 2] = k4.z; kr[r + 3] = k4.w;
         qr[r] = q4.x; qr[r + 1] = q4.y; qr[r + 2] = q4.z; qr[r + 3] = q4.w;
+      }
+      if (CH) {                                     // rows decay one by one, before anything reads them
+#pragma unroll
+        for (int r = 0; r < DR; r += 4) {
+          const float4 g4 = *reinterpret_cast<const float4*>(g_lds + i * DP + row0 + r);
+          s[r] *= g4.x; s[r + 1] *= g4.y; s[r + 2] *= g4.z; s[r + 3] *= g4.w;
+        }
       }
       const float beta = bd_lds[i * 2], dec = bd_lds[i * 2 + 1];
       const float vv = v_lds[i * kWave + lane];
@@ -371,9 +428,11 @@ __global__ __launch_bounds__(256) void gated_delta_rule_kernel(DeltaRuleParams p
 }
 
 template <int DR>
-static void delta_rule_launch(const DeltaRuleParams& p, dim3 grid, hipStream_t s) {
-  const size_t shm = sizeof(float) * (2 * kDeltaChunk * 4 * DR + 2 * kDeltaChunk * kWave + kDeltaChunk * 2 + 4 * 4 * kWave);
-  gated_delta_rule_kernel<DR><<<grid, dim3(256), shm, s>>>(p);
+static void delta_rule_launch(const DeltaRuleParams& p, dim3 grid, hipStream_t s, bool per_channel) {
+  const size_t shm = sizeof(float) * ((per_channel ? 3 : 2) * kDeltaChunk * 4 * DR + 2 * kDeltaChunk * kWave +
+                                      kDeltaChunk * 2 + 4 * 4 * kWave);
+  if (per_channel) gated_delta_rule_kernel<DR, true><<<grid, dim3(256), shm, s>>>(p);
+  else gated_delta_rule_kernel<DR, false><<<grid, dim3(256), shm, s>>>(p);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -381,7 +440,7 @@ template <typename T>
 __global__ __launch_bounds__(256) void head_norm_gate_kernel(const float* __restrict__ o, const T* __restrict__ gate,
                                                              int64_t ld_gate, const float* __restrict__ norm_w,
                                                              T* __restrict__ out, int64_t items, int H, int Dv,
-                                                             float eps) {
+                                                             float eps, int gate_act) {
   const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
   const int64_t item = static_cast<int64_t>(blockIdx.x) * (blockDim.x / kWave) + wave;   // (token, head)
   if (item >= items) return;
@@ -394,7 +453,7 @@ __global__ __launch_bounds__(256) void head_norm_gate_kernel(const float* __rest
   const float inv = 1.0f / sqrtf(ss / static_cast<float>(Dv) + eps);
   for (int e = lane; e < Dv; e += kWave) {
     const float gv = ldf(gate + t * ld_gate + h * Dv + e);
-    stf(out + item * Dv + e, row[e] * inv * norm_w[e] * siluf_(gv));
+    stf(out + item * Dv + e, row[e] * inv * norm_w[e] * (gate_act == LV_MIX_GATE_SILU ? siluf_(gv) : sigmoidf_(gv)));
   }
 }
 
@@ -423,6 +482,27 @@ int lv_hc_update_norm(void* x, const void* y, const void* mix, const void* out_w
   return fail(-1, "lv_hc_update_norm: dtype %d", dtype);
 }
 
+int lv_residual_add_norm(void* x, const void* y1, const void* y2, const void* w, float w_offset, void* out, int64_t T,
+                         int W, float eps, int dtype, void* stream) {
+  if (T == 0) return 0;
+  if (x == nullptr || T < 0 || W <= 0 || (out != nullptr && w == nullptr)) return fail(-1, "lv_residual_add_norm: bad arguments");
+  if (out == nullptr && y1 == nullptr && y2 == nullptr) return 0;
+  const size_t shm = static_cast<size_t>(W + 4) * sizeof(float);
+  if (shm > 64 * 1024) return fail(-2, "lv_residual_add_norm: width %d too large", W);
+  dim3 grid(static_cast<unsigned>(T)), block(256);
+  if (dtype == LV_MIX_BF16)
+    residual_add_norm_kernel<bf16_t><<<grid, block, shm, as_stream(stream)>>>(
+        static_cast<float*>(x), static_cast<const bf16_t*>(y1), static_cast<const bf16_t*>(y2),
+        static_cast<const float*>(w), w_offset, static_cast<bf16_t*>(out), W, eps);
+  else if (dtype == LV_MIX_F32)
+    residual_add_norm_kernel<float><<<grid, block, shm, as_stream(stream)>>>(
+        static_cast<float*>(x), static_cast<const float*>(y1), static_cast<const float*>(y2),
+        static_cast<const float*>(w), w_offset, static_cast<float*>(out), W, eps);
+  else
+    return fail(-1, "lv_residual_add_norm: dtype %d", dtype);
+  return launched("lv_residual_add_norm");
+}
+
 int lv_clamped_glu(const void* in, int64_t ld_in, void* out, int64_t T, int F, float limit, float alpha, int dtype,
                    void* stream) {
   if (T == 0) return 0;
@@ -448,19 +528,22 @@ int lv_clamped_glu(const void* in, int64_t ld_in, void* out, int64_t T, int F, f
 int lv_delta_prep(const void* proj, int64_t ld, const void* conv_w, const void* conv_state, const void* A_log,
                   const void* dt_bias, const int32_t* cu_q, const int32_t* ctx_lens, const int32_t* slots,
                   const int32_t* tok_seq, void* qn, void* kn, void* v, void* beta, void* decay, int64_t T, int G,
-                  int H, int D, int Dv, int taps, int off_b, int off_a, float unit_eps, int dtype, void* stream) {
+                  int H, int D, int Dv, int taps, int off_b, const void* a, int64_t ld_a, int decay_per_channel,
+                  float unit_eps, int dtype, void* stream) {
   if (T == 0) return 0;
   if (!proj || !conv_w || (!conv_state && taps > 1) || !A_log || !dt_bias || !cu_q || !ctx_lens || !slots || !tok_seq || !qn ||
-      !kn || !v || !beta || !decay)
+      !kn || !v || !beta || !decay || !a)
     return fail(-1, "lv_delta_prep: null pointer");
   if (G <= 0 || H <= 0 || H % G != 0 || D <= 0 || Dv <= 0 || taps < 1) return fail(-1, "lv_delta_prep: bad sizes");
   const int C = 2 * G * D + H * Dv;
-  if (ld < C || off_b + H > ld || off_a + H > ld) return fail(-1, "lv_delta_prep: row stride %lld too small", (long long)ld);
+  const int dec_dim = decay_per_channel ? D : 1;
+  if (ld < C || off_b + H > ld || ld_a < static_cast<int64_t>(H) * dec_dim)
+    return fail(-1, "lv_delta_prep: row stride %lld / %lld too small", (long long)ld, (long long)ld_a);
   DeltaPrepParams p{proj, ld, static_cast<const float*>(conv_w), conv_state, static_cast<const float*>(A_log),
                     static_cast<const float*>(dt_bias), cu_q, ctx_lens, slots, tok_seq, static_cast<float*>(qn),
                     static_cast<float*>(kn), static_cast<float*>(v), static_cast<float*>(beta),
-                    static_cast<float*>(decay), T, G, H, D, Dv, taps, off_b, off_a, unit_eps};
-  const int units = 2 * G + H + 1;
+                    static_cast<float*>(decay), T, G, H, D, Dv, taps, off_b, unit_eps, a, ld_a, dec_dim};
+  const int units = 2 * G + H + 1 + (dec_dim > 1 ? H : 0);
   dim3 grid(static_cast<unsigned>(T), (units + 3) / 4), block(256);
   if (dtype == LV_MIX_BF16) delta_prep_kernel<bf16_t><<<grid, block, 0, as_stream(stream)>>>(p);
   else if (dtype == LV_MIX_F32) delta_prep_kernel<float><<<grid, block, 0, as_stream(stream)>>>(p);
@@ -487,7 +570,7 @@ int lv_conv_state_update(const void* proj, int64_t ld, void* conv_state, const i
 
 int lv_gated_delta_rule(const void* qn, const void* kn, const void* v, const void* beta, const void* decay, void* state,
                         const int32_t* cu_q, const int32_t* ctx_lens, const int32_t* slots, void* o, int B, int G,
-                        int H, int D, int Dv, void* stream) {
+                        int H, int D, int Dv, int decay_per_channel, void* stream) {
   if (B == 0) return 0;
   if (!qn || !kn || !v || !beta || !decay || !state || !cu_q || !ctx_lens || !slots || !o)
     return fail(-1, "lv_gated_delta_rule: null pointer");
@@ -498,28 +581,30 @@ int lv_gated_delta_rule(const void* qn, const void* kn, const void* v, const voi
                     cu_q, ctx_lens, slots, static_cast<float*>(o), G, H, D, Dv};
   dim3 grid((Dv + kWave - 1) / kWave, H, B);
   hipStream_t s = as_stream(stream);
-  if (D <= 32) delta_rule_launch<8>(p, grid, s);
-  else if (D <= 64) delta_rule_launch<16>(p, grid, s);
-  else if (D <= 128) delta_rule_launch<32>(p, grid, s);
-  else delta_rule_launch<64>(p, grid, s);
+  const bool ch = decay_per_channel != 0;
+  if (D <= 32) delta_rule_launch<8>(p, grid, s, ch);
+  else if (D <= 64) delta_rule_launch<16>(p, grid, s, ch);
+  else if (D <= 128) delta_rule_launch<32>(p, grid, s, ch);
+  else delta_rule_launch<64>(p, grid, s, ch);
   return launched("lv_gated_delta_rule");
 }
 
 int lv_head_norm_gate(const void* o, const void* gate, int64_t ld_gate, const void* norm_w, void* out, int64_t T,
-                      int H, int Dv, float eps, int dtype, void* stream) {
+                      int H, int Dv, float eps, int gate_act, int dtype, void* stream) {
   if (T == 0) return 0;
-  if (!o || !gate || !norm_w || !out || T < 0 || H <= 0 || Dv <= 0 || ld_gate < static_cast<int64_t>(H) * Dv)
+  if (!o || !gate || !norm_w || !out || T < 0 || H <= 0 || Dv <= 0 || ld_gate < static_cast<int64_t>(H) * Dv ||
+      (gate_act != LV_MIX_GATE_SILU && gate_act != LV_MIX_GATE_SIGMOID))
     return fail(-1, "lv_head_norm_gate: bad arguments");
   const int64_t items = T * H;
   dim3 grid(static_cast<unsigned>((items + 3) / 4)), block(256);
   if (dtype == LV_MIX_BF16)
     head_norm_gate_kernel<bf16_t><<<grid, block, 0, as_stream(stream)>>>(
         static_cast<const float*>(o), static_cast<const bf16_t*>(gate), ld_gate, static_cast<const float*>(norm_w),
-        static_cast<bf16_t*>(out), items, H, Dv, eps);
+        static_cast<bf16_t*>(out), items, H, Dv, eps, gate_act);
   else if (dtype == LV_MIX_F32)
     head_norm_gate_kernel<float><<<grid, block, 0, as_stream(stream)>>>(
         static_cast<const float*>(o), static_cast<const float*>(gate), ld_gate, static_cast<const float*>(norm_w),
-        static_cast<float*>(out), items, H, Dv, eps);
+        static_cast<float*>(out), items, H, Dv, eps, gate_act);
   else
     return fail(-1, "lv_head_norm_gate: dtype %d", dtype);
   return launched("lv_head_norm_gate");

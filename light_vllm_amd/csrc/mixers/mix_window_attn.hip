@@ -83,6 +83,8 @@ struct WindowAttnParams {
   const int32_t *cu_q, *ctx_lens, *tok_seq, *block_tables;
   int bt_stride, H, G, D, Dv, page, window, P, PP;
   float scale, sink;
+  int64_t k_ld, v_ld;   // elements between the rows of two cached tokens (G*D and G*Dv unless the caches are views of wider rows)
+  float m0;             // where the running maximum starts: the sink's score 0, or far below any score without a sink
 };
 
 constexpr int kMaxRep = 8;      // query heads of one kv head served by one workgroup
@@ -123,7 +125,7 @@ __global__ __launch_bounds__(256) void window_pool_attn_kernel(WindowAttnParams 
   float m[kMaxRep], l[kMaxRep], o[kMaxRep][kMaxDvi];
 #pragma unroll
   for (int h = 0; h < kMaxRep; ++h) {
-    m[h] = 0.0f;                                        // never below the sink's score
+    m[h] = p.m0;                                        // with a sink: never below its score
     l[h] = wave == 0 ? p.sink : 0.0f;
 #pragma unroll
     for (int e = 0; e < kMaxDvi; ++e) o[h][e] = 0.0f;
@@ -141,7 +143,7 @@ __global__ __launch_bounds__(256) void window_pool_attn_kernel(WindowAttnParams 
         krow = kpool + (static_cast<int64_t>(bt[pj]) * p.PP + (idx - (p.page * pj) / p.P)) * GD + g * D;
       } else {
         const int j = j0 + idx - nb;
-        krow = kc + (static_cast<int64_t>(bt[j / p.page]) * p.page + j % p.page) * GD + g * D;
+        krow = kc + (static_cast<int64_t>(bt[j / p.page]) * p.page + j % p.page) * p.k_ld + g * D;
       }
     }
     float s[kMaxRep];
@@ -179,7 +181,7 @@ __global__ __launch_bounds__(256) void window_pool_attn_kernel(WindowAttnParams 
         vrow = vpool + (static_cast<int64_t>(bt[pj]) * p.PP + (id2 - (p.page * pj) / p.P)) * GDv + g * Dv;
       } else {
         const int j = j0 + id2 - nb;
-        vrow = vc + (static_cast<int64_t>(bt[j / p.page]) * p.page + j % p.page) * GDv + g * Dv;
+        vrow = vc + (static_cast<int64_t>(bt[j / p.page]) * p.page + j % p.page) * p.v_ld + g * Dv;
       }
 #pragma unroll
       for (int x = 0; x < kMaxDvi; ++x) {
@@ -213,7 +215,7 @@ __global__ __launch_bounds__(256) void window_pool_attn_kernel(WindowAttnParams 
   const T* gate = p.gate != nullptr ? static_cast<const T*>(p.gate) + t * p.ld_gate : nullptr;
   for (int i = threadIdx.x; i < rep * Dv; i += blockDim.x) {
     const int h = i / Dv, dv = i - h * Dv;
-    float mm = 0.0f;
+    float mm = p.m0;
     for (int w = 0; w < 4; ++w) mm = fmaxf(mm, ml_lds[(w * kMaxRep + h) * 2]);
     float ll = 0.0f, acc = 0.0f;
     for (int w = 0; w < 4; ++w) {
@@ -285,10 +287,14 @@ int lv_pool_update(const void* k_cache, const void* v_cache, void* kp, void* vp,
 int lv_window_pool_attn(const void* q, const void* k_cache, const void* v_cache, const void* kp, const void* vp,
                         const void* gate, int64_t ld_gate, void* out, const int32_t* cu_q, const int32_t* ctx_lens,
                         const int32_t* tok_seq, const int32_t* block_tables, int bt_stride, int64_t T, int H, int G, int D,
-                        int Dv, int page, int window, int P, float scale, int has_sink, int dtype, void* stream) {
+                        int Dv, int page, int window, int P, float scale, int has_sink, int64_t k_ld, int64_t v_ld,
+                        int dtype, void* stream) {
   if (T == 0) return 0;
   if (!q || !k_cache || !v_cache || !out || !cu_q || !ctx_lens || !tok_seq || !block_tables)
     return fail(-1, "lv_window_pool_attn: null pointer");
+  if (k_ld <= 0) k_ld = static_cast<int64_t>(G) * D;
+  if (v_ld <= 0) v_ld = static_cast<int64_t>(G) * Dv;
+  if (k_ld < static_cast<int64_t>(G) * D || v_ld < static_cast<int64_t>(G) * Dv) return fail(-1, "lv_window_pool_attn: row strides");
   if (P > 0 && (!kp || !vp)) return fail(-1, "lv_window_pool_attn: pooled blocks without their cache");
   if (T < 0 || H <= 0 || G <= 0 || H % G != 0 || D <= 0 || Dv <= 0 || page <= 0 || window <= 0 || bt_stride <= 0)
     return fail(-1, "lv_window_pool_attn: bad sizes");
@@ -296,7 +302,7 @@ int lv_window_pool_attn(const void* q, const void* k_cache, const void* v_cache,
   const int rep = H / G;
   WindowAttnParams p{q, k_cache, v_cache, kp, vp, gate, ld_gate, out, cu_q, ctx_lens, tok_seq, block_tables,
                      bt_stride, H, G, D, Dv, page, window, P, P > 0 ? (page + P - 1) / P : 0, scale,
-                     has_sink ? 1.0f : 0.0f};
+                     has_sink ? 1.0f : 0.0f, k_ld, v_ld, has_sink ? 0.0f : -1e30f};
   const size_t shm = sizeof(float) * (static_cast<size_t>(kMaxRep) * D + 4 * kMaxRep * kWave +
                                       4 * static_cast<size_t>(kMaxRep) * Dv + 4 * kMaxRep * 2);
   if (shm > 64 * 1024) return fail(-2, "lv_window_pool_attn: head sizes %d / %d need %zu bytes of LDS", D, Dv, shm);

@@ -32,6 +32,8 @@ struct WindowMfmaParams {
   uint32_t m_page, m_P, m_nseg;   // floor(2^32 / d) of the three divisors the tile loop divides by (see fdiv)
   int nsplit;          // > 1 (launches of at most one query tile per sequence): grid.x = split of the key tiles
   float* ws;           // [T, H, nsplit, Dv + 4] partial read-outs, running maximum and sum
+  int64_t k_ld, v_ld;  // elements between the rows of two cached tokens (G*D, G*Dv unless the caches are views of wider rows)
+  float m0;            // start of the running maximum: the sink's score 0, or far below any score without a sink
 };
 
 constexpr int kTileQ = 16;
@@ -109,7 +111,7 @@ __global__ __launch_bounds__(256, (AHEAD || DVB > 8) ? 1 : 4) void window_pool_m
   f32x4_t acc_o[DVB];
 #pragma unroll
   for (int d = 0; d < DVB; ++d) acc_o[d] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
-  float m = 0.0f, l = split == 0 ? p.sink : 0.0f;
+  float m = p.m0, l = split == 0 ? p.sink : 0.0f;
 
   const int nbmax = (P > 0 && i1 - W + 1 > 0) ? (i1 - W + 1) / P : 0;      // pooled blocks the last query sees
   const int jlo = max(0, i0 - W + 1);
@@ -132,8 +134,8 @@ __global__ __launch_bounds__(256, (AHEAD || DVB > 8) ? 1 : 4) void window_pool_m
       const int ec = min(e, i1);
       const int pj = fdiv(ec, page, p.m_page);
       const int64_t slot = static_cast<int64_t>(bt(pj)) * page + (ec - pj * page);
-      kr_ = p.k_cache + slot * GD + g * D;
-      vr_ = p.v_cache + slot * GDv + g * Dv;
+      kr_ = p.k_cache + slot * p.k_ld + g * D;
+      vr_ = p.v_cache + slot * p.v_ld + g * Dv;
     }
   };
   auto tile_start = [&](int tile) { return tile < npt ? tile * kTileK : jlo + (tile - npt) * kTileK; };
@@ -322,14 +324,14 @@ __global__ __launch_bounds__(256, (AHEAD || DVB > 8) ? 1 : 4) void window_pool_m
 // One wave per (token, query head): combines the splits' partials (each with its own running maximum), applies the gate.
 __global__ __launch_bounds__(256) void window_pool_merge_kernel(const float* __restrict__ ws, const uint16_t* __restrict__ gate,
                                                                 int64_t ld_gate, uint16_t* __restrict__ out, int64_t items,
-                                                                int H, int Dv, int nsplit) {
+                                                                int H, int Dv, int nsplit, float m0) {
   const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
   const int64_t item = static_cast<int64_t>(blockIdx.x) * (blockDim.x / kWave) + wave;
   if (item >= items) return;
   const int64_t t = item / H;
   const int h = static_cast<int>(item - t * H);
   const float* w = ws + item * nsplit * (Dv + 4);
-  float mm = 0.0f;
+  float mm = m0;
   for (int s = 0; s < nsplit; ++s) mm = fmaxf(mm, w[s * (Dv + 4) + Dv]);
   float ll = 0.0f;
   for (int s = 0; s < nsplit; ++s) ll += w[s * (Dv + 4) + Dv + 1] * expf(w[s * (Dv + 4) + Dv] - mm);
@@ -354,7 +356,8 @@ extern "C" int lv_window_pool_attn_mfma(const void* q, const void* k_cache, cons
                                         const void* vp, const void* gate, int64_t ld_gate, void* out, const int32_t* cu_q,
                                         const int32_t* ctx_lens, const int32_t* block_tables, int bt_stride, int B,
                                         int max_new_tokens, int H, int G, int D, int Dv, int page, int window, int P,
-                                        float scale, int has_sink, int nsplit, void* workspace, int64_t T, void* stream) {
+                                        float scale, int has_sink, int nsplit, void* workspace, int64_t T, int64_t k_ld,
+                                        int64_t v_ld, void* stream) {
   if (B == 0 || max_new_tokens <= 0) return 0;
   if (!q || !k_cache || !v_cache || !out || !cu_q || !ctx_lens || !block_tables)
     return fail(-1, "lv_window_pool_attn_mfma: null pointer");
@@ -364,6 +367,12 @@ extern "C" int lv_window_pool_attn_mfma(const void* q, const void* k_cache, cons
   if (D % 16 != 0 || Dv % 16 != 0 || D <= 0 || Dv <= 0 || D > 32 * kMaxK32 || Dv > 16 * kMaxDvb)
     return fail(-2, "lv_window_pool_attn_mfma: head sizes %d / %d (multiples of 16 up to 256)", D, Dv);
   if (gate != nullptr && ld_gate < static_cast<int64_t>(H) * Dv) return fail(-1, "lv_window_pool_attn_mfma: gate stride");
+  if (k_ld <= 0) k_ld = static_cast<int64_t>(G) * D;
+  if (v_ld <= 0) v_ld = static_cast<int64_t>(G) * Dv;
+  if (k_ld < static_cast<int64_t>(G) * D || v_ld < static_cast<int64_t>(G) * Dv || k_ld % 8 != 0 || v_ld % 4 != 0 ||
+      (reinterpret_cast<uintptr_t>(k_cache) & 15) != 0 || (reinterpret_cast<uintptr_t>(v_cache) & 7) != 0)
+    return fail(-1, "lv_window_pool_attn_mfma: row strides or alignment of the caches");
+  const float m0 = has_sink ? 0.0f : -1e30f;
   const int rep = H / G;
   const int ngroups = (rep + 3) / 4;
   WindowMfmaParams p{static_cast<const uint16_t*>(q), static_cast<const uint16_t*>(k_cache),
@@ -371,7 +380,8 @@ extern "C" int lv_window_pool_attn_mfma(const void* q, const void* k_cache, cons
                      static_cast<const uint16_t*>(vp), static_cast<const uint16_t*>(gate), ld_gate,
                      static_cast<uint16_t*>(out), cu_q, ctx_lens, block_tables, bt_stride, H, G, D, Dv, page, window, P,
                      P > 0 ? (page + P - 1) / P : 0, ngroups, scale, has_sink ? 1.0f : 0.0f,
-                     magic(page), magic(P > 0 ? P : 1), magic(Dv / 4), nsplit > 1 ? nsplit : 1, static_cast<float*>(workspace)};
+                     magic(page), magic(P > 0 ? P : 1), magic(Dv / 4), nsplit > 1 ? nsplit : 1, static_cast<float*>(workspace),
+                     k_ld, v_ld, m0};
   if (nsplit > 1 && (max_new_tokens > kTileQ || workspace == nullptr || T <= 0))
     return fail(-1, "lv_window_pool_attn_mfma: key splits need one query tile per sequence and a workspace");
   const size_t shm = static_cast<size_t>(Dv) * kLdk * sizeof(uint16_t);
@@ -389,7 +399,7 @@ extern "C" int lv_window_pool_attn_mfma(const void* q, const void* k_cache, cons
     const int64_t items = T * H;
     window_pool_merge_kernel<<<dim3(static_cast<unsigned>((items + 3) / 4)), block, 0, st>>>(
         static_cast<const float*>(workspace), static_cast<const uint16_t*>(gate), ld_gate, static_cast<uint16_t*>(out),
-        items, H, Dv, nsplit);
+        items, H, Dv, nsplit, m0);
   }
   return launched("lv_window_pool_attn_mfma");
 }

@@ -1,12 +1,13 @@
 """RMSNorm and fused residual-add + RMSNorm with the reference's rounding points
 (lightvllm/layers/layernorm.py:28-80): fp32 math, one rounding to the activation dtype before the
-weight multiply, the new residual rounded once from the fp32 sum."""
+weight multiply, the new residual rounded once from the fp32 sum. OffsetRMSNorm: the norm of models
+that keep their residual in f32 and hold the norm weight as an offset from one."""
 from __future__ import annotations
 
 import torch
 from torch import nn
 
-from .. import ops
+from .. import mix_ops, ops
 from .fused import use_fused
 
 
@@ -40,3 +41,17 @@ class RMSNorm(nn.Module):
         if residual is None:
             return self.rms_forward(x)
         return self.add_rms_forward(x, residual)
+
+
+class OffsetRMSNorm(nn.Module):
+    """x / sqrt(mean(x^2) + eps) * (offset + w) on an f32 residual, fused with the residual update that
+    precedes it: `forward(x, y1, y2)` adds up to two sublayer outputs to x in place and returns the normed
+    row in the activation dtype (mix_ops.residual_add_norm, one launch). The weight is f32."""
+
+    def __init__(self, hidden_size: int, eps: float = 1e-6, offset: float = 1.0):
+        super().__init__()
+        self.hidden_size, self.eps, self.offset = hidden_size, eps, float(offset)
+        self.weight = nn.Parameter(torch.zeros(hidden_size, dtype=torch.float32))
+
+    def forward(self, x: torch.Tensor, y1=None, y2=None, act_dtype=None) -> torch.Tensor:
+        return mix_ops.residual_add_norm(x, y1, y2, self.weight, self.offset, self.eps, act_dtype)

@@ -1,0 +1,52 @@
+"""Mixture-of-experts feed-forward: `experts` small two-matrix feed-forward layers, of which each token
+uses `top`, chosen by a sigmoid router.
+
+    s = sigmoid(W_r h) (32-bit)          selection scores c = s + correction (the correction steers the
+    selection only); the experts are split into `groups` consecutive blocks, a block is ranked by the sum of its two
+    largest c, experts outside the `keep` highest-ranked blocks are excluded, and the `top` largest c that remain win.
+    weights = s of the chosen / (their sum + 1e-20)      y = sum_chosen weight_e * W_down,e act(W_up,e h)
+
+act is the squared relu. All experts' up matrices are one [experts * ff, width] weight and all down
+matrices one [width, experts * ff] weight. The step computes the up projection of every expert in one
+GEMM, then one kernel applies the activation times the token's weight for the column's expert (zero for
+experts the token did not choose), and the down GEMM sums over experts by itself: two vendor GEMMs and two
+small launches, no host synchronisation, capturable into a hipGraph. It spends experts / top times the
+FLOPs a gathered form would.
+"""
+from __future__ import annotations
+
+import torch
+import torch.nn.functional as F
+from torch import nn
+
+from .. import mix_ops
+from .tp import tp_size
+
+
+class SparseMoE(nn.Module):
+
+    def __init__(self, width: int, ff: int, experts: int, top: int, groups: int = 1, keep: int = 1,
+                 share: "SparseMoE | None" = None):
+        super().__init__()
+        assert tp_size() == 1, "the mixture of experts is not sharded: run it with tensor_parallel_size 1"
+        assert 1 <= top <= experts and groups >= 1 and experts % groups == 0 and 1 <= keep <= groups
+        self.width, self.ff, self.E, self.top, self.groups, self.keep = width, ff, experts, top, groups, keep
+        if share is None:
+            f32 = dict(dtype=torch.float32)
+            self.router_weight = nn.Parameter(torch.empty(experts, width, **f32))
+            self.correction = nn.Parameter(torch.zeros(experts, **f32))
+            self.up_weight = nn.Parameter(torch.empty(experts * ff, width))
+            self.down_weight = nn.Parameter(torch.empty(width, experts * ff))
+        else:
+            assert (share.width, share.ff, share.E) == (width, ff, experts)
+            self.router_weight, self.correction = share.router_weight, share.correction
+            self.up_weight, self.down_weight = share.up_weight, share.down_weight
+
+    def route(self, h: torch.Tensor):
+        logits = F.linear(h.float(), self.router_weight)
+        return mix_ops.moe_route(logits, self.correction, self.top, self.groups, self.keep)
+
+    def forward(self, h: torch.Tensor) -> torch.Tensor:
+        _, _, dense = self.route(h)
+        up = F.linear(h, self.up_weight)
+        return F.linear(mix_ops.relu2_scale(up, dense, self.E, self.ff), self.down_weight)

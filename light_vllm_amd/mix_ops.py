@@ -60,6 +60,32 @@ def hc_update_norm(x, y=None, mix=None, out_w=None, in_w=None, norm_w=None, grou
     return out
 
 
+def residual_add_norm(x, y1=None, y2=None, w=None, w_offset=0.0, eps=1e-6, act_dtype=None):
+    """x [T, W] f32 (the one residual) += y1 + y2 in place (either may be None); returns
+    x / sqrt(mean(x^2) + eps) * (w_offset + w) in act dtype, or None when w is None."""
+    T, W = x.shape
+    _f32(x, w)
+    ys = [y for y in (y1, y2) if y is not None]
+    act_dtype = act_dtype or (ys[0].dtype if ys else torch.bfloat16)
+    out = torch.empty(T, W, dtype=act_dtype, device=x.device) if w is not None else None
+    if x.is_cuda:
+        for y in ys:
+            assert y.is_contiguous() and y.dtype == act_dtype and y.shape == (T, W)
+        lib = _mixlib.load()
+        _mixlib.check(lib.lv_residual_add_norm(_p(x), _p(y1), _p(y2), _p(w), w_offset, _p(out), T, W, eps, _DT[act_dtype],
+                                               _stream(x)), "lv_residual_add_norm")
+        return out
+    if ys:
+        add = ys[0].float()
+        if len(ys) > 1:
+            add = add + ys[1].float()
+        x.add_(add)
+    if w is None:
+        return None
+    out.copy_(x / torch.sqrt(x.pow(2).mean(-1, keepdim=True) + eps) * (w_offset + w))
+    return out
+
+
 def clamped_glu(x, limit: float, alpha: float):
     """x [T, 2F] = [gate | up] -> min(g, L) * sigmoid(alpha * g) * (clamp(u, -L, L) + 1), [T, F]."""
     T, F2 = x.shape
@@ -78,28 +104,34 @@ def clamped_glu(x, limit: float, alpha: float):
 
 
 # ------------------------------------------------------------------------------------- delta rule
-def delta_prep(proj, conv_w, conv_state, A_log, dt_bias, step, G, H, D, Dv, taps, off_b, off_a, unit_eps):
+def delta_prep(proj, conv_w, conv_state, A_log, dt_bias, step, G, H, D, Dv, taps, off_b, a, unit_eps,
+               decay_per_channel=False):
     """Short causal convolution + silu over the q | k | v channels of `proj` [T, ld] (taps from the
     portion's own rows, then from the carried state of the sequence's slot, zeros before position
     0), unit-norm q (times D^-1/2) and k per head, beta = sigmoid(b), decay = exp(-exp(A_log) *
-    softplus(a + dt_bias)). Returns f32 (qn [T,G,D], kn [T,G,D], v [T,H,Dv], beta [T,H], decay [T,H])."""
+    softplus(a + dt_bias)) with a [T, H] (a view of proj's columns or a tensor of its own), or
+    [T, H*D] with decay_per_channel (dt_bias [H*D], A_log [H]).
+    Returns f32 (qn [T,G,D], kn [T,G,D], v [T,H,Dv], beta [T,H], decay [T,H] or [T,H,D])."""
     T = proj.size(0)
     dev = proj.device
     _f32(conv_w, A_log, dt_bias)
+    nd = D if decay_per_channel else 1
+    assert a.shape == (T, H * nd) and a.dtype == proj.dtype and dt_bias.numel() == H * nd
     qn = torch.empty(T, G, D, dtype=torch.float32, device=dev)
     kn = torch.empty(T, G, D, dtype=torch.float32, device=dev)
     v = torch.empty(T, H, Dv, dtype=torch.float32, device=dev)
     beta = torch.empty(T, H, dtype=torch.float32, device=dev)
-    decay = torch.empty(T, H, dtype=torch.float32, device=dev)
+    decay = torch.empty((T, H, D) if decay_per_channel else (T, H), dtype=torch.float32, device=dev)
     C = 2 * G * D + H * Dv
     assert conv_state.is_contiguous() and conv_state.shape[1:] == (taps - 1, C) and conv_state.dtype == proj.dtype
     if proj.is_cuda:
-        assert proj.stride(1) == 1
+        assert proj.stride(1) == 1 and a.stride(1) == 1
         lib = _mixlib.load()
         _mixlib.check(lib.lv_delta_prep(_p(proj), proj.stride(0), _p(conv_w), _p(conv_state), _p(A_log), _p(dt_bias),
                                         _p(step.cu_q), _p(step.ctx_lens), _p(step.slots), _p(step.tok_seq), _p(qn),
-                                        _p(kn), _p(v), _p(beta), _p(decay), T, G, H, D, Dv, taps, off_b, off_a,
-                                        unit_eps, _DT[proj.dtype], _stream(proj)), "lv_delta_prep")
+                                        _p(kn), _p(v), _p(beta), _p(decay), T, G, H, D, Dv, taps, off_b, _p(a),
+                                        a.stride(0), int(decay_per_channel), unit_eps, _DT[proj.dtype], _stream(proj)),
+                      "lv_delta_prep")
         return qn, kn, v, beta, decay
     q0 = 0
     for b, (n, ctx) in enumerate(zip(step.host_lens_q, step.host_ctx_lens)):
@@ -117,7 +149,12 @@ def delta_prep(proj, conv_w, conv_state, A_log, dt_bias, step, G, H, D, Dv, taps
         kn[q0:q0 + n] = kk / torch.sqrt(kk.pow(2).sum(-1, keepdim=True) + unit_eps)
         v[q0:q0 + n] = y[:, 2 * G * D:].view(n, H, Dv)
         beta[q0:q0 + n] = torch.sigmoid(proj[q0:q0 + n, off_b:off_b + H].float())
-        decay[q0:q0 + n] = torch.exp(-torch.exp(A_log) * F.softplus(proj[q0:q0 + n, off_a:off_a + H].float() + dt_bias))
+        sp = F.softplus(a[q0:q0 + n].float() + dt_bias.view(-1))
+        rate = torch.exp(A_log)
+        if decay_per_channel:
+            decay[q0:q0 + n] = torch.exp(-rate[None, :, None] * sp.view(n, H, D))
+        else:
+            decay[q0:q0 + n] = torch.exp(-rate * sp)
         q0 += n
     return qn, kn, v, beta, decay
 
@@ -145,18 +182,21 @@ def conv_state_update(proj, conv_state, step, C, taps):
 
 def gated_delta_rule(qn, kn, v, beta, decay, state, step):
     """Per head and token: S <- decay * S; u = beta * (v - S^T k); S <- S + k u^T; o = S^T q.
+    decay [T, H] scales a head's whole state, decay [T, H, D] each of its rows (key channels) by its own number.
     state f32 [slots, H, D, Dv] (taken as zero for a sequence with no context), updated in place.
     Returns o f32 [T, H, Dv]."""
     T, G, D = qn.shape
     H, Dv = v.shape[1], v.shape[2]
     _f32(qn, kn, v, beta, decay, state)
     assert state.shape[1:] == (H, D, Dv)
+    per_channel = decay.dim() == 3
+    assert decay.shape == ((T, H, D) if per_channel else (T, H))
     o = torch.empty(T, H, Dv, dtype=torch.float32, device=qn.device)
     if qn.is_cuda:
         lib = _mixlib.load()
         _mixlib.check(lib.lv_gated_delta_rule(_p(qn), _p(kn), _p(v), _p(beta), _p(decay), _p(state), _p(step.cu_q),
                                               _p(step.ctx_lens), _p(step.slots), _p(o), len(step.host_lens_q), G, H, D,
-                                              Dv, _stream(qn)), "lv_gated_delta_rule")
+                                              Dv, int(per_channel), _stream(qn)), "lv_gated_delta_rule")
         return o
     rep = H // G
     q0 = 0
@@ -166,7 +206,7 @@ def gated_delta_rule(qn, kn, v, beta, decay, state, step):
         for t in range(q0, q0 + n):
             k = kn[t].repeat_interleave(rep, 0)      # [H, D]
             q = qn[t].repeat_interleave(rep, 0)
-            S = decay[t][:, None, None] * S
+            S = (decay[t][:, :, None] if per_channel else decay[t][:, None, None]) * S
             u = beta[t][:, None] * (v[t] - torch.einsum("hdv,hd->hv", S, k))
             S = S + k[:, :, None] * u[:, None, :]
             o[t] = torch.einsum("hdv,hd->hv", S, q)
@@ -175,8 +215,10 @@ def gated_delta_rule(qn, kn, v, beta, decay, state, step):
     return o
 
 
-def head_norm_gate(o, gate, norm_w, eps, act_dtype):
-    """o f32 [T, H, Dv] -> act [T, H*Dv]: per-head RMS norm over Dv, times norm_w [Dv], times silu(gate)."""
+def head_norm_gate(o, gate, norm_w, eps, act_dtype, gate_act="silu"):
+    """o f32 [T, H, Dv] -> act [T, H*Dv]: per-head RMS norm over Dv, times norm_w [Dv], times silu(gate)
+    or sigmoid(gate)."""
+    assert gate_act in ("silu", "sigmoid")
     T, H, Dv = o.shape
     _f32(o, norm_w)
     out = torch.empty(T, H * Dv, dtype=act_dtype, device=o.device)
@@ -184,10 +226,11 @@ def head_norm_gate(o, gate, norm_w, eps, act_dtype):
         assert gate.stride(1) == 1 and gate.dtype == act_dtype
         lib = _mixlib.load()
         _mixlib.check(lib.lv_head_norm_gate(_p(o), _p(gate), gate.stride(0), _p(norm_w), _p(out), T, H, Dv, eps,
-                                            _DT[act_dtype], _stream(o)), "lv_head_norm_gate")
+                                            int(gate_act == "sigmoid"), _DT[act_dtype], _stream(o)), "lv_head_norm_gate")
         return out
     y = o / torch.sqrt(o.pow(2).mean(-1, keepdim=True) + eps) * norm_w
-    out.copy_((y * F.silu(gate.float()).view(T, H, Dv)).reshape(T, H * Dv))
+    g = F.silu(gate.float()) if gate_act == "silu" else torch.sigmoid(gate.float())
+    out.copy_((y * g.view(T, H, Dv)).reshape(T, H * Dv))
     return out
 
 
@@ -271,15 +314,21 @@ def window_pool_attention(q, k_cache, v_cache, kp, vp, gate, step, H, G, D, Dv, 
     """Query at position i attends to cached positions j with 0 <= i - j < window and to the pooled
     entry of every block b with b*P + P - 1 <= i - window, one softmax over both, `has_sink` adding 1
     to its denominator; the result is multiplied by sigmoid(gate) when a gate is given.
-    q [T, H*D] contiguous act; returns act [T, H*Dv]."""
+    q [T, H*D] contiguous act; returns act [T, H*Dv]. k_cache and v_cache [pages, page, G, D|Dv] may be
+    views of wider token rows (one cache row serving as key and, in part, as value). A window that no
+    sequence reaches, no pool and no sink give plain causal softmax attention."""
     T = q.size(0)
     page = k_cache.size(1)
     out = torch.empty(T, H * Dv, dtype=q.dtype, device=q.device)
+    k_ld, v_ld = k_cache.stride(1), v_cache.stride(1)
     if q.is_cuda:
         assert q.is_contiguous() and (gate is None or gate.stride(1) == 1)
+        for c, ld, d in ((k_cache, k_ld, D), (v_cache, v_ld, Dv)):
+            assert c.stride(3) == 1 and (G == 1 or c.stride(2) == d) and c.stride(0) == page * ld and ld >= G * d
         lib = _mixlib.load()
         if (WINDOW_ATTN_KERNEL == "auto" and q.dtype == torch.bfloat16 and D % 16 == 0 and Dv % 16 == 0
-                and D <= 256 and Dv <= 256):
+                and D <= 256 and Dv <= 256 and k_ld % 8 == 0 and v_ld % 4 == 0 and k_cache.data_ptr() % 16 == 0
+                and v_cache.data_ptr() % 8 == 0):
             # decode-shaped steps put one workgroup per (sequence, kv head) on the chip: cut each sequence's key
             # tiles over enough workgroups to fill it (partials merged by a second kernel)
             nsplit, ws = 1, None
@@ -295,18 +344,18 @@ def window_pool_attention(q, k_cache, v_cache, kp, vp, gate, step, H, G, D, Dv, 
                                                        _p(step.ctx_lens), _p(step.block_tables),
                                                        step.block_tables.stride(0), len(step.host_lens_q),
                                                        max(step.host_lens_q), H, G, D, Dv, page, window, P, scale,
-                                                       int(has_sink), nsplit, _p(ws), T, _stream(q)),
+                                                       int(has_sink), nsplit, _p(ws), T, k_ld, v_ld, _stream(q)),
                           "lv_window_pool_attn_mfma")
             return out
         _mixlib.check(lib.lv_window_pool_attn(_p(q), _p(k_cache), _p(v_cache), _p(kp), _p(vp), _p(gate),
                                               gate.stride(0) if gate is not None else 0, _p(out), _p(step.cu_q),
                                               _p(step.ctx_lens), _p(step.tok_seq), _p(step.block_tables),
                                               step.block_tables.stride(0), T, H, G, D, Dv, page, window, P, scale,
-                                              int(has_sink), _DT[q.dtype], _stream(q)), "lv_window_pool_attn")
+                                              int(has_sink), k_ld, v_ld, _DT[q.dtype], _stream(q)), "lv_window_pool_attn")
         return out
     PP = pooled_slots(page, P)
     rep = H // G
-    kc, vc = k_cache.view(-1, G, D), v_cache.view(-1, G, Dv)
+    kc, vc = k_cache.reshape(-1, G, D), v_cache.reshape(-1, G, Dv)
     q0 = 0
     for b, (n, ctx) in enumerate(zip(step.host_lens_q, step.host_ctx_lens)):
         bt = step.host_block_tables[b]
@@ -321,7 +370,9 @@ def window_pool_attention(q, k_cache, v_cache, kp, vp, gate, step, H, G, D, Dv, 
                 V = torch.cat([vp.view(-1, G, Dv)[prow].float(), V])
             qi = q[q0 + r].float().view(G, rep, D)
             s = torch.einsum("grd,ngd->grn", qi, K) * scale
-            m = s.max(-1, keepdim=True).values.clamp(min=0)
+            m = s.max(-1, keepdim=True).values
+            if has_sink:
+                m = m.clamp(min=0)
             e = torch.exp(s - m)
             w = e / (e.sum(-1, keepdim=True) + (torch.exp(-m) if has_sink else 0))
             o = torch.einsum("grn,ngv->grv", w, V).reshape(H * Dv)
@@ -329,4 +380,145 @@ def window_pool_attention(q, k_cache, v_cache, kp, vp, gate, step, H, G, D, Dv, 
                 o = o * torch.sigmoid(gate[q0 + r].float())
             out[q0 + r] = o
         q0 += n
+    return out
+
+
+# ------------------------------------------------------------------------------- latent attention
+def rotary_inv_freq(dims: int, base: float, device) -> torch.Tensor:
+    """f32 [dims/2]: base^(-2i/dims), computed in 64-bit and rounded once."""
+    i = torch.arange(dims // 2, dtype=torch.float64)
+    return torch.pow(torch.tensor(float(base), dtype=torch.float64), -2.0 * i / dims).float().to(device)
+
+
+def _rotate(x, pos, inv_freq, dims):
+    """x f32 [n, ..., d]: the first `dims` entries rotated pairwise (i, i + dims/2) by pos * inv_freq[i]."""
+    if dims == 0:
+        return x
+    half = dims // 2
+    ang = pos.float().view(-1, *([1] * (x.dim() - 1))) * inv_freq.view(*([1] * (x.dim() - 1)), half)
+    c, s = torch.cos(ang), torch.sin(ang)
+    u, v = x[..., :half], x[..., half:dims]
+    return torch.cat([u * c - v * s, v * c + u * s, x[..., dims:]], -1)
+
+
+def _positions(step, device):
+    return torch.cat([torch.arange(c, c + n, device=device) for n, c in zip(step.host_lens_q, step.host_ctx_lens)])
+
+
+def latent_prep(proj, off_q, off_kv, q_w, kv_w, inv_freq, cache, step, Rq, R, Dr, rot_dims, eps):
+    """proj [T, ld]: query latent at column off_q (Rq wide), key/value latent at off_kv (R wide) followed
+    by the positional key part (Dr wide). Returns the RMS-normed query latent [T, Rq]; writes
+    [rms_norm(latent) * kv_w | rotated positional part] into each token's row of cache [pages, page, R + Dr]."""
+    T = proj.size(0)
+    page = cache.size(1)
+    _f32(q_w, kv_w, inv_freq)
+    cq = torch.empty(T, Rq, dtype=proj.dtype, device=proj.device)
+    assert cache.is_contiguous() and cache.shape[2] == R + Dr and cache.dtype == proj.dtype
+    if proj.is_cuda:
+        assert proj.stride(1) == 1
+        lib = _mixlib.load()
+        _mixlib.check(lib.lv_latent_prep(_p(proj), proj.stride(0), off_q, off_kv, _p(q_w), _p(kv_w), _p(inv_freq), _p(cq),
+                                         _p(cache), _p(step.cu_q), _p(step.ctx_lens), _p(step.tok_seq),
+                                         _p(step.block_tables), step.block_tables.stride(0), T, Rq, R, Dr, rot_dims, page,
+                                         eps, _DT[proj.dtype], _stream(proj)), "lv_latent_prep")
+        return cq
+    x = proj[:, off_q:off_q + Rq].float()
+    cq.copy_(x / torch.sqrt(x.pow(2).mean(-1, keepdim=True) + eps) * q_w)
+    c = proj[:, off_kv:off_kv + R].float()
+    c = c / torch.sqrt(c.pow(2).mean(-1, keepdim=True) + eps) * kv_w
+    pos = _positions(step, proj.device)
+    kr = _rotate(proj[:, off_kv + R:off_kv + R + Dr].float(), pos, inv_freq, rot_dims)
+    rows = torch.cat([c, kr], -1).to(cache.dtype)
+    flat = cache.view(-1, R + Dr)
+    q0 = 0
+    for b, (n, ctx) in enumerate(zip(step.host_lens_q, step.host_ctx_lens)):
+        bt = step.host_block_tables[b]
+        for r in range(n):
+            flat[_token_slot(bt, ctx + r, page)] = rows[q0 + r]
+        q0 += n
+    return cq
+
+
+def latent_q_finish(q, q_lat, inv_freq, step, H, Dn, Dr, R, rot_dims):
+    """q [T, H*(Dn+Dr)] (per head: Dn unrotated entries, then Dr to rotate), q_lat [H, T, R] (the unrotated
+    part multiplied into the latent space) -> [T, H*(R+Dr)] = per head [q_lat | rotated part]."""
+    T = q.size(0)
+    out = torch.empty(T, H * (R + Dr), dtype=q.dtype, device=q.device)
+    assert q.is_contiguous() and q_lat.is_contiguous() and q_lat.shape == (H, T, R)
+    if q.is_cuda:
+        _f32(inv_freq)
+        lib = _mixlib.load()
+        _mixlib.check(lib.lv_latent_q_finish(_p(q), _p(q_lat), _p(inv_freq), _p(out), _p(step.cu_q), _p(step.ctx_lens),
+                                             _p(step.tok_seq), T, H, Dn, Dr, R, rot_dims, _DT[q.dtype], _stream(q)),
+                      "lv_latent_q_finish")
+        return out
+    o = out.view(T, H, R + Dr)
+    o[:, :, :R] = q_lat.transpose(0, 1)
+    if Dr:
+        qr = q.view(T, H, Dn + Dr)[:, :, Dn:].float()
+        o[:, :, R:] = _rotate(qr, _positions(step, q.device), inv_freq, rot_dims).to(q.dtype)
+    return out
+
+
+def latent_out_gate(o, gate, per_channel: bool):
+    """o [H, T, Dv] -> [T, H*Dv] times sigmoid(gate); gate [T, H] (one per head) or [T, H*Dv]."""
+    H, T, Dv = o.shape
+    out = torch.empty(T, H * Dv, dtype=o.dtype, device=o.device)
+    assert gate.shape == (T, H * Dv if per_channel else H) and gate.dtype == o.dtype
+    if o.is_cuda:
+        assert o.is_contiguous() and gate.stride(1) == 1
+        lib = _mixlib.load()
+        _mixlib.check(lib.lv_latent_out_gate(_p(o), _p(gate), gate.stride(0), int(per_channel), _p(out), T, H, Dv,
+                                             _DT[o.dtype], _stream(o)), "lv_latent_out_gate")
+        return out
+    g = torch.sigmoid(gate.float())
+    g = g.view(T, H, Dv) if per_channel else g.view(T, H, 1)
+    out.copy_((o.float().transpose(0, 1) * g).reshape(T, H * Dv))
+    return out
+
+
+# ------------------------------------------------------------------------------ mixture of experts
+def moe_route(logits, correction, top, groups=1, keep=1):
+    """logits f32 [T, E] -> (ids int32 [T, top], weights f32 [T, top], dense f32 [T, E]).
+    Scores s = sigmoid(logits); the choice goes by s + correction; with `groups` > 1 only experts of the
+    `keep` blocks of consecutive experts ranked highest by the sum of their two top selection scores stay in the selection; weights are the
+    chosen s over their sum (+ 1e-20); dense holds them at the chosen experts and 0 elsewhere."""
+    T, E = logits.shape
+    _f32(logits, correction)
+    dev = logits.device
+    ids = torch.empty(T, top, dtype=torch.int32, device=dev)
+    w = torch.empty(T, top, dtype=torch.float32, device=dev)
+    dense = torch.empty(T, E, dtype=torch.float32, device=dev)
+    if logits.is_cuda:
+        lib = _mixlib.load()
+        _mixlib.check(lib.lv_moe_route(_p(logits), _p(correction), _p(ids), _p(w), _p(dense), T, E, top, groups, keep,
+                                       _stream(logits)), "lv_moe_route")
+        return ids, w, dense
+    s = torch.sigmoid(logits)
+    c = s + correction if correction is not None else s.clone()
+    if groups > 1 and keep < groups:
+        cg = c.view(T, groups, E // groups)
+        gs = cg.topk(min(2, E // groups), -1).values.sum(-1)
+        best = gs.topk(keep, -1).indices
+        kept = torch.zeros(T, groups, dtype=torch.bool).scatter_(1, best, True)
+        c = cg.masked_fill(~kept[:, :, None], float("-inf")).reshape(T, E)
+    idx = c.topk(top, -1).indices
+    ws = s.gather(1, idx)
+    ws = ws / (ws.sum(-1, keepdim=True) + 1e-20)
+    ids.copy_(idx)
+    w.copy_(ws)
+    dense.zero_().scatter_(1, idx, ws)
+    return ids, w, dense
+
+
+def relu2_scale(up, dense, E, Fe):
+    """up act [T, E*Fe] (all experts' up projections), dense f32 [T, E] -> relu(up)^2 * dense[t, e], act."""
+    T = up.size(0)
+    out = torch.empty_like(up)
+    if up.is_cuda:
+        assert up.is_contiguous() and dense.is_contiguous() and dense.dtype == torch.float32
+        lib = _mixlib.load()
+        _mixlib.check(lib.lv_relu2_scale(_p(up), _p(dense), _p(out), T, E, Fe, _DT[up.dtype], _stream(up)), "lv_relu2_scale")
+        return out
+    out.copy_((torch.relu(up.float()).pow(2).view(T, E, Fe) * dense[:, :, None]).reshape(T, E * Fe))
     return out

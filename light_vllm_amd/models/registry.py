@@ -21,9 +21,15 @@ def _kagalorn():
     return KagalornForCausalLM
 
 
+def _bokulorn():
+    from .bokulorn import BokulornForCausalLM
+    return BokulornForCausalLM
+
+
 MODELS = {
     "Qwen3ForCausalLM": _qwen3,
     "Kagalorn": _kagalorn,
+    "Bokulorn": _bokulorn,
 }
 DEFAULT = "Qwen3ForCausalLM"
 

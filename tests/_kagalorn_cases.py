@@ -105,7 +105,7 @@ def case_delta_rule_portions(device, dtype):
             proj = torch.cat(rows).to(device)
             qn, kn, v, beta, dec = mix_ops.delta_prep(proj, conv_w.to(device), conv_state, A_log.to(device),
                                                       dt_bias.to(device), step, G, H, D, Dv, taps, C + H * Dv,
-                                                      C + H * Dv + H, 1e-6)
+                                                      proj[:, C + H * Dv + H:C + H * Dv + 2 * H], 1e-6)
             mix_ops.conv_state_update(proj, conv_state, step, C, taps)
             o = mix_ops.gated_delta_rule(qn, kn, v, beta, dec, state, step).cpu()
             got0.append(o[:n0])
