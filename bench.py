@@ -720,6 +720,171 @@ def _mixer_kernel_table(z, dev, batch, prompt_len):
     return rows
 
 
+# --mixers-design bokulorn: the Bokulorn design (latent attention, channel-wise delta rule, mixture-of-experts
+# feed-forwards on one f32 residual) beside Kagalorn, the closest existing model (ragged steps, a delta rule and an
+# attention over a paged cache), at equal width, depth, head counts and active feed-forward size.
+BOKULORN_SIZES = {
+    "2k": dict(q_rank=768, kv_rank=192, rot_dim=64, experts=32, top=4, groups=4, keep=2, thin=64),
+    "4k": dict(q_rank=1536, kv_rank=192, rot_dim=64, experts=32, top=4, groups=4, keep=2, thin=128),
+}
+
+
+def _bokulorn_config(z, bz):
+    from light_vllm_amd.models.bokulorn import BokulornConfig
+    H, D = z["heads"], z["dim"]
+    lat = {"heads": H, "dim": D, "vdim": D, "q_rank": bz["q_rank"], "kv_rank": bz["kv_rank"], "rot_dim": bz["rot_dim"],
+           "rot": {"base": 10000.0, "dims": bz["rot_dim"]}, "scale": (D + bz["rot_dim"]) ** -0.5}
+    lat2 = {"heads": H, "dim": D, "vdim": D, "q_rank": bz["q_rank"], "kv_rank": bz["kv_rank"] + bz["rot_dim"], "scale": D ** -0.5}
+    dlt = {"heads": H, "kv_heads": z["kv_heads"], "dim": D, "vdim": D, "conv": 4, "decay_rank": bz["thin"], "gate_rank": bz["thin"]}
+    mlp = {"kind": "moe", "expert": {"ff": z["ff"] // bz["top"]},
+           "router": {"experts": bz["experts"], "top": bz["top"], "groups": {"count": bz["groups"], "keep": bz["keep"]}}}
+    kinds = [("channel_delta", dlt), ("latent_attention", lat), ("channel_delta", dlt), ("latent_attention_2", lat2)]
+    layers = [{"type": kinds[i % 4][0], "mixer": kinds[i % 4][1], "mlp": mlp} for i in range(z["layers"])]
+    return BokulornConfig.from_dict({"vocab": z["vocab"], "width": z["width"], "norm": {"eps": 1e-6},
+                                     "embedding": {"scale": z["width"] ** 0.5}, "layers": layers})
+
+
+def _bokulorn_kernel_table(z, bz, dev, batch, prompt_len):
+    """Each kernel of the design alone at one layer's shapes (prompt step and decode step), beside the Kagalorn
+    kernel that does the like job."""
+    from light_vllm_amd import mix_ops
+    from light_vllm_amd.layers.latent_attention import NO_WINDOW
+    from light_vllm_amd.layers.moe import SparseMoE
+    from light_vllm_amd.utils.context import RaggedStep
+    bf = torch.bfloat16
+    W, H, G, D = z["width"], z["heads"], z["kv_heads"], z["dim"]
+    R, Dr, Rq, E, top = bz["kv_rank"], bz["rot_dim"], bz["q_rank"], bz["experts"], bz["top"]
+    Fe = z["ff"] // top
+    page = 256
+    rows = []
+
+    def step_of(lens_q, ctx):
+        B = len(lens_q)
+        cu, tok = [0], []
+        for b, n_ in enumerate(lens_q):
+            cu.append(cu[-1] + n_)
+            tok += [b] * n_
+        per = -(-(max(ctx) + max(lens_q)) // page)
+        tables = [[b * per + j for j in range(per)] for b in range(B)]
+        i32 = dict(dtype=torch.int32, device=dev)
+        return RaggedStep(torch.tensor(cu, **i32), torch.tensor(ctx, **i32), torch.arange(B, **i32),
+                          torch.tensor(tok, **i32), torch.tensor(tables, **i32), lens_q, ctx, list(range(B)), tables), B * per
+
+    def add(name, phase, fn, nbytes=0, flops=0, like=None):
+        us = _event_time(fn, 20, 3) * 1e6
+        rec = {"kernel": name, "phase": phase, "us": round(us, 1)}
+        if nbytes:
+            rec["of_hbm_roofline"] = round(nbytes / us / 1e3 / (HBM_BPS / 1e9), 3)
+        if flops:
+            rec["TFLOPs"] = round(flops / us / 1e6, 2)
+            rec["of_mfma_roofline"] = round(flops / us / 1e6 / (MFMA_FLOPS / 1e12), 4)
+        if like:
+            rec["like"] = like
+        rows.append(rec)
+
+    old_default = torch.get_default_dtype()
+    torch.set_default_dtype(bf)
+    try:
+        moe = SparseMoE(W, Fe, E, top, bz["groups"], bz["keep"]).to(dev)
+    finally:
+        torch.set_default_dtype(old_default)
+    for prm in moe.parameters():
+        prm.data.normal_(0.0, 0.02)
+    for phase, lens_q, ctx in (("prompt", [prompt_len] * batch, [0] * batch), ("decode", [1] * batch, [prompt_len] * batch)):
+        step, pages = step_of(lens_q, ctx)
+        T = sum(lens_q)
+        x = torch.randn(T, W, device=dev)
+        y1, y2 = torch.randn(T, W, device=dev, dtype=bf), torch.randn(T, W, device=dev, dtype=bf)
+        nw = torch.zeros(W, device=dev)
+        add("residual_add_norm", phase, lambda: mix_ops.residual_add_norm(x, y1, y2, nw, 1.0, 1e-6, bf), nbytes=T * W * 14)
+        xs = torch.randn(T, 4, W, device=dev)
+        mixm, vec = torch.eye(4, device=dev), torch.ones(4, device=dev)
+        add("kagalorn hc_update_norm", phase, lambda: mix_ops.hc_update_norm(xs, y1, mixm, vec, vec, nw, 4, 1e-6, bf),
+            nbytes=T * W * 36, like="residual_add_norm")
+        # latent attention
+        proj = torch.randn(T, Rq + R + Dr + H, device=dev, dtype=bf)
+        inv_freq = mix_ops.rotary_inv_freq(Dr, 10000.0, dev)
+        cache = torch.zeros(pages, page, R + Dr, device=dev, dtype=bf)
+        qw, kw_ = torch.ones(Rq, device=dev), torch.ones(R, device=dev)
+        add("latent_prep", phase, lambda: mix_ops.latent_prep(proj, 0, Rq, qw, kw_, inv_freq, cache, step, Rq, R, Dr, Dr, 1e-6),
+            nbytes=T * (Rq * 4 + (R + Dr) * 4))
+        q = torch.randn(T, H * (D + Dr), device=dev, dtype=bf)
+        q_lat = torch.randn(H, T, R, device=dev, dtype=bf)
+        add("latent_q_finish", phase, lambda: mix_ops.latent_q_finish(q, q_lat, inv_freq, step, H, D, Dr, R, Dr),
+            nbytes=T * H * ((R + Dr) * 4))
+        q_abs = mix_ops.latent_q_finish(q, q_lat, inv_freq, step, H, D, Dr, R, Dr)
+        kc = cache.unsqueeze(2)
+        keys = sum(i + 1 for n_, c0 in zip(lens_q, ctx) for i in range(c0, c0 + n_))
+        attn = lambda: mix_ops.window_pool_attention(q_abs, kc, kc[..., :R], None, None, None, step, H, 1, R + Dr, R,  # noqa: E731
+                                                     NO_WINDOW, 0, 0.07, has_sink=False)
+        if phase == "prompt":
+            add("latent attention", phase, attn, flops=keys * H * (2 * R + Dr) * 2)
+        else:
+            add("latent attention", phase, attn, nbytes=keys * (R + Dr) * 2)
+        o = torch.randn(H, T, D, device=dev, dtype=bf)
+        add("latent_out_gate", phase, lambda: mix_ops.latent_out_gate(o, proj[:, Rq + R + Dr:], False), nbytes=T * H * D * 4)
+        # the like kernel: windowed pooled attention of Kagalorn with the window open to the whole context
+        kq = torch.randn(T, H * D, device=dev, dtype=bf)
+        kk = torch.zeros(pages, page, G, D, device=dev, dtype=bf)
+        kattn = lambda: mix_ops.window_pool_attention(kq, kk, kk, None, None, None, step, H, G, D, D, NO_WINDOW, 0,  # noqa: E731
+                                                      D ** -0.5, True)
+        if phase == "prompt":
+            add("kagalorn window_pool_attn", phase, kattn, flops=keys * H * D * 4, like="latent attention")
+        else:
+            add("kagalorn window_pool_attn", phase, kattn, nbytes=keys * G * D * 4, like="latent attention")
+        # channel-wise delta rule
+        C = 2 * G * D + H * D
+        dproj = torch.randn(T, C + H, device=dev, dtype=bf)
+        a = torch.randn(T, H * D, device=dev, dtype=bf)
+        conv_w = torch.randn(C, 4, device=dev) * 0.5
+        conv_state = torch.zeros(batch, 3, C, device=dev, dtype=bf)
+        A_log = torch.zeros(H, device=dev)
+        state = torch.zeros(batch, H, D, D, device=dev)
+        for ch in (True, False):
+            dtb = torch.zeros(H * D if ch else H, device=dev)
+            a_in = a if ch else a[:, :H]
+            name = "channel" if ch else "kagalorn per-head"
+            add(f"delta_prep ({name})", phase, lambda: mix_ops.delta_prep(dproj, conv_w, conv_state, A_log, dtb, step, G, H, D, D, 4, C,
+                                                                         a_in, 1e-6, decay_per_channel=ch),
+                nbytes=T * (C * 6 + (H * D * 6 if ch else 0)), like=None if ch else "delta_prep (channel)")
+            qn, kn, v, beta, dec = mix_ops.delta_prep(dproj, conv_w, conv_state, A_log, dtb, step, G, H, D, D, 4, C, a_in, 1e-6,
+                                                      decay_per_channel=ch)
+            add(f"gated_delta_rule ({name})", phase, lambda: mix_ops.gated_delta_rule(qn, kn, v, beta, dec, state, step),
+                nbytes=batch * H * D * D * 8 + T * (2 * G * D + 2 * H * D + (H * D if ch else 0)) * 4,
+                like=None if ch else "gated_delta_rule (channel)")
+        # mixture of experts
+        h = torch.randn(T, W, device=dev, dtype=bf)
+        logits = torch.randn(T, E, device=dev)
+        add("moe_route", phase, lambda: mix_ops.moe_route(logits, moe.correction, top, bz["groups"], bz["keep"]))
+        with torch.inference_mode():
+            add("moe feed-forward (all of it)", phase, lambda: moe(h), flops=T * top * Fe * W * 4)
+            wg = torch.randn(2 * z["ff"], W, device=dev, dtype=bf) * 0.02
+            wd = torch.randn(W, z["ff"], device=dev, dtype=bf) * 0.02
+            add("kagalorn dense feed-forward", phase,
+                lambda: torch.nn.functional.linear(mix_ops.clamped_glu(torch.nn.functional.linear(h, wg), 7.0, 1.702), wd),
+                flops=T * z["ff"] * W * 6, like="moe feed-forward (all of it)")
+    return rows
+
+
+def bokulorn_leg(sizes, batch, prompt_len, new_tokens):
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    out = {"metric": "mixers: Bokulorn beside Kagalorn at equal size", "dtype": "bf16", "data": "synthetic, random weights",
+           "batch": batch, "prompt_len": prompt_len, "new_tokens": new_tokens, "sizes": []}
+    for name in sizes:
+        z, bz = MIXER_SIZES[name], BOKULORN_SIZES[name]
+        rec = {"size": name, **z, **bz}
+        cache_tokens = batch * 256 * (-(-(prompt_len + new_tokens) // 256))
+        kw = dict(kvcache_block_size=256, max_cache_tokens=cache_tokens)
+        rec["bokulorn"] = _engine_rates(_bokulorn_config(z, bz), batch, prompt_len, new_tokens, **kw)
+        rec["bokulorn_graph"] = _engine_rates(_bokulorn_config(z, bz), batch, prompt_len, new_tokens, enforce_eager=False, **kw)
+        rec["kagalorn"] = _engine_rates(_kagalorn_config(z), batch, prompt_len, new_tokens, **kw)
+        rec["kagalorn_graph"] = _engine_rates(_kagalorn_config(z), batch, prompt_len, new_tokens, enforce_eager=False, **kw)
+        rec["kernels"] = _bokulorn_kernel_table(z, bz, dev, batch, prompt_len)
+        out["sizes"].append(rec)
+    print(json.dumps(out), flush=True)
+
+
 def mixers_leg(sizes, batch, prompt_len, new_tokens):
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
@@ -791,10 +956,14 @@ def main():
                          "(proves launcher, rendezvous, graph and JSON path; not a measurement)")
     ap.add_argument("--mixers", default="", help="comma list of sizes (2k, 4k): instead of the default workload, "
                     "run the Kagalorn design beside Qwen3 at equal size and time its kernels one by one")
+    ap.add_argument("--mixers-design", default="kagalorn", choices=("kagalorn", "bokulorn"),
+                    help="with --mixers: kagalorn (beside Qwen3) or bokulorn (beside Kagalorn, its closest relative)")
     ap.add_argument("--mixers-batch", type=int, default=16)
     ap.add_argument("--mixers-prompt", type=int, default=1024)
     ap.add_argument("--mixers-new", type=int, default=17)
     args = ap.parse_args()
+    if args.mixers and args.mixers_design == "bokulorn":
+        return bokulorn_leg([x for x in args.mixers.split(",") if x], args.mixers_batch, args.mixers_prompt, args.mixers_new)
     if args.mixers:
         return mixers_leg([x for x in args.mixers.split(",") if x], args.mixers_batch, args.mixers_prompt, args.mixers_new)
 

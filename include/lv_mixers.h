@@ -23,6 +23,7 @@
  *   lv_latent_out_gate       per-head outputs [H, T, Dv] -> [T, H*Dv] times sigmoid(gate), gate per head or per channel
  *   lv_moe_route             sigmoid router with a selection-only correction, group limit and top-k
  *   lv_relu2_scale           squared relu of the experts' up projections times the routing weight
+ *   lv_moe_grouped_ff        the experts' feed-forward on rows sorted by expert (grouped GEMMs on the matrix cores)
  *
  * A "ragged step" is a batch of B sequences; sequence b brings cu_q[b+1]-cu_q[b] new tokens that
  * follow ctx_lens[b] tokens already in the cache / state (a whole prompt, a portion of one, or one
@@ -168,6 +169,15 @@ int lv_moe_route(const void* logits, const void* correction, void* ids, void* we
 /* up act [T, E*F] (all experts' up projections side by side), dense f32 [T, E]:
  * out act [T, E*F] = relu(up)^2 * dense[t, e]. */
 int lv_relu2_scale(const void* up, const void* dense, void* out, int64_t T, int E, int F, int dtype, void* stream);
+
+/* The gathered form of the same feed-forward, bf16 only, W and F multiples of 32: the (token, choice) pairs are sorted by
+ * expert on the device, each expert multiplies its own rows on the matrix cores (up projection with relu^2, down
+ * projection), and every token sums its choices' rows times their weights in f32. Four launches, no host round trip.
+ * h bf16 [T, W]; ids int32 [T, top]; weights f32 [T, top]; up_w bf16 [E*F, W]; down_w bf16 [W, E*F]; out bf16 [T, W];
+ * workspace: lv_moe_grouped_workspace_bytes(T, W, F, E, top) bytes, 16-byte aligned. */
+int lv_moe_grouped_ff(const void* h, const void* ids, const void* weights, const void* up_w, const void* down_w, void* out,
+                      void* workspace, int64_t T, int W, int F, int E, int top, void* stream);
+int64_t lv_moe_grouped_workspace_bytes(int64_t T, int W, int F, int E, int top);
 
 #ifdef __cplusplus
 }

@@ -16,7 +16,7 @@ from ctypes import c_char_p, c_float, c_int, c_int64, c_void_p
 _HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(_HERE, "csrc", "mixers")
 LIB_PATH = os.path.join(_HERE, "lib", "liblvmix.so")
-SOURCES = ["mix_stream.hip", "mix_window_attn.hip", "mix_window_mfma.hip", "mix_latent.hip"]
+SOURCES = ["mix_stream.hip", "mix_window_attn.hip", "mix_window_mfma.hip", "mix_latent.hip", "mix_moe_gemm.hip"]
 ABI_VERSION = 5
 
 _P = c_void_p
@@ -46,6 +46,8 @@ SIGNATURES = {
     "lv_latent_out_gate": (c_int, [_P, _P, c_int64, c_int, _P, c_int64, c_int, c_int, c_int, _P]),
     "lv_moe_route": (c_int, [_P, _P, _P, _P, _P, c_int64, c_int, c_int, c_int, c_int, _P]),
     "lv_relu2_scale": (c_int, [_P, _P, _P, c_int64, c_int, c_int, c_int, _P]),
+    "lv_moe_grouped_ff": (c_int, [_P, _P, _P, _P, _P, _P, _P, c_int64, c_int, c_int, c_int, c_int, _P]),
+    "lv_moe_grouped_workspace_bytes": (c_int64, [c_int64, c_int, c_int, c_int, c_int]),
 }
 
 _lib = None

@@ -1,0 +1,239 @@
+// Mixture of experts, gathered form, for bf16: tokens are sorted by expert on the device and every expert multiplies
+// only its own rows.
+//
+//   moe_sort_kernel      one workgroup: counts the (token, choice) pairs of every expert, gives each pair a row in
+//                        expert order, and lists the row tiles (expert, first row, rows) that the GEMM launches walk.
+//                        No host round trip: the GEMM grids are sized for the most tiles a step can have and
+//                        workgroups beyond the list leave at once.
+//   moe_gemm_kernel      grouped GEMM on the matrix cores, one workgroup per (row tile of one expert, column tile):
+//                        C[row, n] = sum_k A[row, k] * B_e[n, k], both operands with k contiguous, so MFMA fragments
+//                        (v_mfma_f32_16x16x32_bf16) are 16-byte loads straight from memory; the four waves share the
+//                        tile's rows and split its columns. The weights are the MFMA's first operand: a lane then holds
+//                        four consecutive columns of one row and stores them as 8 bytes.
+//                        UP: rows are gathered from the tokens' activations, epilogue relu(x)^2.
+//                        DOWN: rows are the sorted activations, B_e is a column block of the one [width, experts*ff] weight.
+//   moe_combine_kernel   one workgroup per token: sum over its choices of weight * expert output row, in f32.
+// A row's result does not depend on where the sort put it or on what else is in the tile: every output element is
+// its own chain of MFMA accumulations over k.
+#include "mix_common.h"
+
+namespace lvmix {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
+typedef __attribute__((ext_vector_type(4))) float f32x4_t;
+
+constexpr int kSortThreads = 1024;
+
+// ids [M] (expert of pair p = token * top + choice).  Outputs: sorted_pair [M] (pair of each row in expert order),
+// inv [M] (row of each pair), tiles [max_tiles][3] (expert, first row, rows), num_tiles [1].
+__global__ __launch_bounds__(kSortThreads) void moe_sort_kernel(const int32_t* __restrict__ ids, int M, int E, int BM,
+                                                                 int32_t* __restrict__ sorted_pair, int32_t* __restrict__ inv,
+                                                                 int32_t* __restrict__ tiles, int32_t* __restrict__ num_tiles,
+                                                                 int max_tiles) {
+  extern __shared__ int32_t sl[];
+  int32_t* cnt = sl;              // [E] pairs per expert
+  int32_t* off = sl + E;          // [E + 1] first row per expert
+  int32_t* toff = sl + 2 * E + 1; // [E + 1] first tile per expert
+  for (int e = threadIdx.x; e < E; e += blockDim.x) cnt[e] = 0;
+  __syncthreads();
+  for (int p = threadIdx.x; p < M; p += blockDim.x) inv[p] = atomicAdd(&cnt[ids[p]], 1);     // rank inside the expert
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int r = 0, t = 0;
+    for (int e = 0; e < E; ++e) {
+      off[e] = r;
+      toff[e] = t;
+      r += cnt[e];
+      t += (cnt[e] + BM - 1) / BM;
+    }
+    off[E] = r;
+    toff[E] = t;
+    num_tiles[0] = t < max_tiles ? t : max_tiles;
+  }
+  __syncthreads();
+  for (int p = threadIdx.x; p < M; p += blockDim.x) {
+    const int row = off[ids[p]] + inv[p];
+    sorted_pair[row] = p;
+    inv[p] = row;
+  }
+  for (int e = threadIdx.x; e < E; e += blockDim.x) {
+    const int n = cnt[e];
+    for (int j = 0, t = toff[e]; j * BM < n && t < max_tiles; ++j, ++t) {
+      tiles[3 * t] = e;
+      tiles[3 * t + 1] = off[e] + j * BM;
+      tiles[3 * t + 2] = min(BM, n - j * BM);
+    }
+  }
+}
+
+struct MoeGemmParams {
+  const uint16_t* A;       // UP: activations [T, K]; DOWN: sorted expert activations [M, K]
+  const uint16_t* B;       // UP: [E * N, K]; DOWN: [N, E * K]
+  uint16_t* C;             // [M, N] in sorted row order
+  const int32_t *sorted_pair, *tiles, *num_tiles;
+  int N, K, top;
+  int64_t lda, ldb, ldc;
+  int64_t b_expert;        // elements from one expert's B to the next
+};
+
+// MB x NB blocks of 16 x 16 per wave; the workgroup's tile is (16 MB) rows x (4 * 16 NB) columns.
+template <int MB, int NB, bool UP>
+__global__ __launch_bounds__(256) void moe_gemm_kernel(MoeGemmParams p) {
+  const int tile = blockIdx.y;
+  if (tile >= p.num_tiles[0]) return;
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+  const int ln = lane & 15, lg = lane >> 4;
+  const int e = p.tiles[3 * tile], row0 = p.tiles[3 * tile + 1], nrows = p.tiles[3 * tile + 2];
+  const int n0 = (blockIdx.x * 4 + wave) * 16 * NB;
+  if (n0 >= p.N) return;
+  const uint16_t* arow[MB];
+#pragma unroll
+  for (int mb = 0; mb < MB; ++mb) {
+    const int r = row0 + min(mb * 16 + ln, nrows - 1);          // rows past the tile's end repeat its last row; never stored
+    const int64_t src = UP ? p.sorted_pair[r] / p.top : r;
+    arow[mb] = p.A + src * p.lda + 8 * lg;
+  }
+  const uint16_t* brow[NB];
+#pragma unroll
+  for (int nb = 0; nb < NB; ++nb) {
+    const int n = min(n0 + nb * 16 + ln, p.N - 1);
+    brow[nb] = p.B + static_cast<int64_t>(e) * p.b_expert + static_cast<int64_t>(n) * p.ldb + 8 * lg;
+  }
+  f32x4_t acc[MB][NB];
+#pragma unroll
+  for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) acc[mb][nb] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+  for (int k = 0; k < p.K; k += 32) {
+    bf16x8_t a[MB], b[NB];
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) a[mb] = *reinterpret_cast<const bf16x8_t*>(arow[mb] + k);
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) b[nb] = *reinterpret_cast<const bf16x8_t*>(brow[nb] + k);
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb)
+        acc[mb][nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(b[nb], a[mb], acc[mb][nb], 0, 0, 0);
+  }
+  // acc[mb][nb][i] = C[row = 16 mb + ln][n = n0 + 16 nb + 4 lg + i]
+#pragma unroll
+  for (int mb = 0; mb < MB; ++mb) {
+    const int r = mb * 16 + ln;
+    if (r >= nrows) continue;
+    uint16_t* crow = p.C + static_cast<int64_t>(row0 + r) * p.ldc;
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+      const int n = n0 + nb * 16 + 4 * lg;
+      if (n >= p.N) continue;                                   // N is a multiple of 4: a lane's four columns are in or out together
+      uint16_t o[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        float v = acc[mb][nb][i];
+        if (UP) {
+          v = fmaxf(v, 0.0f);
+          v = v * v;
+        }
+        bf16_t t;
+        stf(&t, v);
+        o[i] = t.bits;
+      }
+      *reinterpret_cast<uint2*>(crow + n) = uint2{static_cast<uint32_t>(o[0]) | (static_cast<uint32_t>(o[1]) << 16),
+                                                  static_cast<uint32_t>(o[2]) | (static_cast<uint32_t>(o[3]) << 16)};
+    }
+  }
+}
+
+__global__ __launch_bounds__(256) void moe_combine_kernel(const uint16_t* __restrict__ rows, const int32_t* __restrict__ inv,
+                                                          const float* __restrict__ weights, uint16_t* __restrict__ out,
+                                                          int W, int top) {
+  const int64_t t = blockIdx.x;
+  for (int c = threadIdx.x * 4; c < W; c += blockDim.x * 4) {
+    float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    for (int k = 0; k < top; ++k) {
+      const float w = weights[t * top + k];
+      const uint2 v = *reinterpret_cast<const uint2*>(rows + static_cast<int64_t>(inv[t * top + k]) * W + c);
+      acc[0] += w * __builtin_bit_cast(float, v.x << 16);
+      acc[1] += w * __builtin_bit_cast(float, v.x & 0xffff0000u);
+      acc[2] += w * __builtin_bit_cast(float, v.y << 16);
+      acc[3] += w * __builtin_bit_cast(float, v.y & 0xffff0000u);
+    }
+    bf16_t o[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) stf(&o[i], acc[i]);
+    *reinterpret_cast<uint2*>(out + t * W + c) = uint2{static_cast<uint32_t>(o[0].bits) | (static_cast<uint32_t>(o[1].bits) << 16),
+                                                        static_cast<uint32_t>(o[2].bits) | (static_cast<uint32_t>(o[3].bits) << 16)};
+  }
+}
+
+template <bool UP>
+static void gemm_launch(const MoeGemmParams& p, int max_tiles, int BM, hipStream_t s) {
+  if (BM == 64) {
+    dim3 grid((p.N + 4 * 64 - 1) / (4 * 64), max_tiles);
+    moe_gemm_kernel<4, 4, UP><<<grid, dim3(256), 0, s>>>(p);
+  } else {
+    dim3 grid((p.N + 4 * 32 - 1) / (4 * 32), max_tiles);
+    moe_gemm_kernel<1, 2, UP><<<grid, dim3(256), 0, s>>>(p);
+  }
+}
+
+}  // namespace lvmix
+
+using namespace lvmix;
+
+extern "C" {
+
+int lv_moe_tile_rows(int64_t pairs, int E) {
+  // few rows per expert (decoded tokens): tiles of 16 rows read each weight once and waste little of the matrix cores;
+  // prompts: 64 rows share every weight fragment
+  return pairs >= static_cast<int64_t>(E) * 48 ? 64 : 16;
+}
+
+int lv_moe_max_tiles(int64_t pairs, int E, int BM) {
+  const int64_t full = pairs / BM + E;            // every expert can end on a partial tile
+  const int64_t hit = pairs < E ? pairs : E;
+  const int64_t most = pairs / BM + hit;
+  return static_cast<int>(most < full ? most : full);
+}
+
+int lv_moe_grouped_ff(const void* h, const void* ids, const void* weights, const void* up_w, const void* down_w, void* out,
+                      void* workspace, int64_t T, int W, int F, int E, int top, void* stream) {
+  if (T == 0) return 0;
+  if (!h || !ids || !weights || !up_w || !down_w || !out || !workspace) return fail(-1, "lv_moe_grouped_ff: null pointer");
+  if (T < 0 || W <= 0 || F <= 0 || E <= 0 || top <= 0 || W % 32 != 0 || F % 32 != 0 || E > 4096)
+    return fail(-1, "lv_moe_grouped_ff: width %d and expert size %d must be multiples of 32 (experts %d)", W, F, E);
+  const int64_t M = T * top;
+  if (M > (1 << 30)) return fail(-2, "lv_moe_grouped_ff: %lld rows", (long long)M);
+  const int BM = lv_moe_tile_rows(M, E);
+  const int max_tiles = lv_moe_max_tiles(M, E, BM);
+  // workspace: sorted_pair [M] | inv [M] | tiles [3 max_tiles] | num_tiles [1] (int32, padded to 16 bytes) | act [M, F] | rows [M, W]
+  int32_t* sorted_pair = static_cast<int32_t*>(workspace);
+  int32_t* inv = sorted_pair + M;
+  int32_t* tiles = inv + M;
+  int32_t* num_tiles = tiles + 3 * static_cast<int64_t>(max_tiles);
+  const int64_t ints = (2 * M + 3 * static_cast<int64_t>(max_tiles) + 1 + 3) / 4 * 4;
+  uint16_t* act = reinterpret_cast<uint16_t*>(sorted_pair + ints);
+  uint16_t* rows = act + M * F;
+  hipStream_t s = as_stream(stream);
+  const size_t shm = sizeof(int32_t) * (3 * static_cast<size_t>(E) + 2);
+  moe_sort_kernel<<<dim3(1), dim3(kSortThreads), shm, s>>>(static_cast<const int32_t*>(ids), static_cast<int>(M), E, BM,
+                                                          sorted_pair, inv, tiles, num_tiles, max_tiles);
+  MoeGemmParams up{static_cast<const uint16_t*>(h), static_cast<const uint16_t*>(up_w), act, sorted_pair, tiles, num_tiles,
+                   F, W, top, W, W, F, static_cast<int64_t>(F) * W};
+  gemm_launch<true>(up, max_tiles, BM, s);
+  MoeGemmParams down{act, static_cast<const uint16_t*>(down_w), rows, sorted_pair, tiles, num_tiles,
+                     W, F, top, F, static_cast<int64_t>(E) * F, W, F};
+  gemm_launch<false>(down, max_tiles, BM, s);
+  moe_combine_kernel<<<dim3(static_cast<unsigned>(T)), dim3(256), 0, s>>>(rows, inv, static_cast<const float*>(weights),
+                                                                          static_cast<uint16_t*>(out), W, top);
+  return launched("lv_moe_grouped_ff");
+}
+
+int64_t lv_moe_grouped_workspace_bytes(int64_t T, int W, int F, int E, int top) {
+  const int64_t M = T * top;
+  const int BM = lv_moe_tile_rows(M, E);
+  const int64_t ints = (2 * M + 3 * static_cast<int64_t>(lv_moe_max_tiles(M, E, BM)) + 1 + 3) / 4 * 4;
+  return ints * 4 + M * (static_cast<int64_t>(F) + W) * 2;
+}
+
+}  // extern "C"

@@ -7,11 +7,17 @@ uses `top`, chosen by a sigmoid router.
     weights = s of the chosen / (their sum + 1e-20)      y = sum_chosen weight_e * W_down,e act(W_up,e h)
 
 act is the squared relu. All experts' up matrices are one [experts * ff, width] weight and all down
-matrices one [width, experts * ff] weight. The step computes the up projection of every expert in one
-GEMM, then one kernel applies the activation times the token's weight for the column's expert (zero for
-experts the token did not choose), and the down GEMM sums over experts by itself: two vendor GEMMs and two
-small launches, no host synchronisation, capturable into a hipGraph. It spends experts / top times the
-FLOPs a gathered form would.
+matrices one [width, experts * ff] weight. Two forms compute the same sum:
+
+  * gathered (bf16, width and ff in multiples of 32, at least GATHER_FROM experts per choice): the (token,
+    choice) pairs are sorted by expert on the device and every expert multiplies only its own rows
+    (mix_ops.moe_grouped_ff: sort, two grouped GEMMs on the matrix cores, weighted sum; four launches);
+  * masked (f32, other sizes, few experts per choice): the up projection of every expert in one vendor
+    GEMM, one kernel applies the activation times the token's weight for the column's expert (zero for
+    experts the token did not choose), and the down GEMM sums over experts by itself. It spends
+    experts / top times the FLOPs of the gathered form.
+
+Neither synchronises with the host, so both can be captured into a hipGraph.
 """
 from __future__ import annotations
 
@@ -21,6 +27,10 @@ from torch import nn
 
 from .. import mix_ops
 from .tp import tp_size
+
+
+GATHER_FROM = 2.0     # experts / top from which the gathered form is taken
+MOE_KERNEL = "auto"   # "auto" | "masked" | "gathered" (tests force one or the other)
 
 
 class SparseMoE(nn.Module):
@@ -46,7 +56,14 @@ class SparseMoE(nn.Module):
         logits = F.linear(h.float(), self.router_weight)
         return mix_ops.moe_route(logits, self.correction, self.top, self.groups, self.keep)
 
+    def gathered(self, h: torch.Tensor) -> bool:
+        if MOE_KERNEL != "auto":
+            return MOE_KERNEL == "gathered"
+        return mix_ops.moe_grouped_ok(h, self.ff) and self.E >= GATHER_FROM * self.top
+
     def forward(self, h: torch.Tensor) -> torch.Tensor:
-        _, _, dense = self.route(h)
+        ids, weights, dense = self.route(h)
+        if self.gathered(h):
+            return mix_ops.moe_grouped_ff(h, ids, weights, self.up_weight, self.down_weight, self.E, self.ff)
         up = F.linear(h, self.up_weight)
         return F.linear(mix_ops.relu2_scale(up, dense, self.E, self.ff), self.down_weight)

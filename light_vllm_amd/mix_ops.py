@@ -522,3 +522,35 @@ def relu2_scale(up, dense, E, Fe):
         return out
     out.copy_((torch.relu(up.float()).pow(2).view(T, E, Fe) * dense[:, :, None]).reshape(T, E * Fe))
     return out
+
+
+def moe_grouped_ok(h, Fe) -> bool:
+    """Whether moe_grouped_ff serves these shapes (bf16, width and expert size in multiples of 32)."""
+    return h.dtype == torch.bfloat16 and h.size(1) % 32 == 0 and Fe % 32 == 0
+
+
+def moe_grouped_ff(h, ids, weights, up_w, down_w, E, Fe):
+    """y[t] = sum_k weights[t, k] * W_down,e relu(W_up,e h[t])^2 with e = ids[t, k], computed expert by expert on rows
+    sorted by expert: up_w [E*Fe, W], down_w [W, E*Fe]. The expert outputs are rounded to the activation dtype
+    before the weighted sum, which is in f32. Returns act [T, W]."""
+    T, W = h.shape
+    top = ids.size(1)
+    out = torch.empty(T, W, dtype=h.dtype, device=h.device)
+    if h.is_cuda:
+        assert moe_grouped_ok(h, Fe) and h.is_contiguous() and up_w.is_contiguous() and down_w.is_contiguous()
+        assert ids.dtype == torch.int32 and ids.is_contiguous() and weights.is_contiguous() and weights.dtype == torch.float32
+        lib = _mixlib.load()
+        ws = torch.empty(lib.lv_moe_grouped_workspace_bytes(T, W, Fe, E, top), dtype=torch.uint8, device=h.device)
+        _mixlib.check(lib.lv_moe_grouped_ff(_p(h), _p(ids), _p(weights), _p(up_w), _p(down_w), _p(out), _p(ws), T, W, Fe, E, top,
+                                            _stream(h)), "lv_moe_grouped_ff")
+        return out
+    acc = torch.zeros(T, W)
+    for e in range(E):
+        t_idx, k_idx = (ids == e).nonzero(as_tuple=True)
+        if t_idx.numel() == 0:
+            continue
+        a = torch.relu(F.linear(h[t_idx], up_w[e * Fe:(e + 1) * Fe]).float()).pow(2).to(h.dtype)
+        y = F.linear(a, down_w[:, e * Fe:(e + 1) * Fe]).float()
+        acc.index_add_(0, t_idx, y * weights[t_idx, k_idx][:, None])
+    out.copy_(acc)
+    return out

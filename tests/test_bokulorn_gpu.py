@@ -64,6 +64,17 @@ def test_matrix_core_attention_agrees_with_the_vector_kernel(gpu, tmp_path):
         mix_ops.WINDOW_ATTN_KERNEL = old
 
 
+def test_masked_experts_serve_the_model_like_the_gathered_ones(gpu, tmp_path):
+    """The bf16 schedules above take the gathered form of the feed-forward (sizes in multiples of 32); here the
+    masked form is forced on the same model."""
+    from light_vllm_amd.layers import moe
+    old, moe.MOE_KERNEL = moe.MOE_KERNEL, "masked"
+    try:
+        C.case_engine_schedules(DEV, "bfloat16", tmp_path, cfg=K.CFG_WIDE, seed=11)
+    finally:
+        moe.MOE_KERNEL = old
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_engine_reuse_of_pages_and_slots(gpu, tmp_path, dtype):
     C.case_engine_reuse(DEV, dtype, tmp_path)
