@@ -76,20 +76,24 @@ struct MoeGemmParams {
   int64_t b_expert;        // elements from one expert's B to the next
 };
 
-// MB x NB blocks of 16 x 16 per wave; the workgroup's tile is (16 MB) rows x (4 * 16 NB) columns.
-template <int MB, int NB, bool UP>
+// MB x NB blocks of 16 x 16 per wave; WM waves along the rows (1 or 2), the others along the columns: the workgroup's
+// tile is (16 MB WM) rows x (16 NB 4 / WM) columns. The fragments of the next 32-wide step over k are loaded before the
+// matrix instructions of the current one are issued, so that memory latency is covered by them.
+template <int MB, int NB, int WM, bool UP>
 __global__ __launch_bounds__(256) void moe_gemm_kernel(MoeGemmParams p) {
-  const int tile = blockIdx.y;
+  const int tile = blockIdx.y, bx = blockIdx.x;
   if (tile >= p.num_tiles[0]) return;
   const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
   const int ln = lane & 15, lg = lane >> 4;
+  const int wm = wave % WM, wn = wave / WM;
   const int e = p.tiles[3 * tile], row0 = p.tiles[3 * tile + 1], nrows = p.tiles[3 * tile + 2];
-  const int n0 = (blockIdx.x * 4 + wave) * 16 * NB;
-  if (n0 >= p.N) return;
+  const int m0 = wm * 16 * MB;
+  const int n0 = (bx * (4 / WM) + wn) * 16 * NB;
+  if (n0 >= p.N || m0 >= nrows) return;
   const uint16_t* arow[MB];
 #pragma unroll
   for (int mb = 0; mb < MB; ++mb) {
-    const int r = row0 + min(mb * 16 + ln, nrows - 1);          // rows past the tile's end repeat its last row; never stored
+    const int r = row0 + min(m0 + mb * 16 + ln, nrows - 1);     // rows past the tile's end repeat its last row; never stored
     const int64_t src = UP ? p.sorted_pair[r] / p.top : r;
     arow[mb] = p.A + src * p.lda + 8 * lg;
   }
@@ -104,22 +108,32 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(MoeGemmParams p) {
   for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb) acc[mb][nb] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
-  for (int k = 0; k < p.K; k += 32) {
-    bf16x8_t a[MB], b[NB];
+  bf16x8_t a0[MB], b0[NB], a1[MB], b1[NB];
+  auto load = [&](bf16x8_t* a, bf16x8_t* b, int k) {
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) a[mb] = *reinterpret_cast<const bf16x8_t*>(arow[mb] + k);
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb) b[nb] = *reinterpret_cast<const bf16x8_t*>(brow[nb] + k);
+  };
+  auto multiply = [&](const bf16x8_t* a, const bf16x8_t* b) {
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
       for (int nb = 0; nb < NB; ++nb)
         acc[mb][nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(b[nb], a[mb], acc[mb][nb], 0, 0, 0);
+  };
+  load(a0, b0, 0);
+  for (int k = 0; k < p.K; k += 64) {
+    if (k + 32 < p.K) load(a1, b1, k + 32);
+    multiply(a0, b0);
+    if (k + 32 >= p.K) break;
+    if (k + 64 < p.K) load(a0, b0, k + 64);
+    multiply(a1, b1);
   }
-  // acc[mb][nb][i] = C[row = 16 mb + ln][n = n0 + 16 nb + 4 lg + i]
+  // acc[mb][nb][i] = C[row = m0 + 16 mb + ln][n = n0 + 16 nb + 4 lg + i]
 #pragma unroll
   for (int mb = 0; mb < MB; ++mb) {
-    const int r = mb * 16 + ln;
+    const int r = m0 + mb * 16 + ln;
     if (r >= nrows) continue;
     uint16_t* crow = p.C + static_cast<int64_t>(row0 + r) * p.ldc;
 #pragma unroll
@@ -168,12 +182,15 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const uint16_t* __rest
 
 template <bool UP>
 static void gemm_launch(const MoeGemmParams& p, int max_tiles, int BM, hipStream_t s) {
-  if (BM == 64) {
-    dim3 grid((p.N + 4 * 64 - 1) / (4 * 64), max_tiles);
-    moe_gemm_kernel<4, 4, UP><<<grid, dim3(256), 0, s>>>(p);
-  } else {
-    dim3 grid((p.N + 4 * 32 - 1) / (4 * 32), max_tiles);
-    moe_gemm_kernel<1, 2, UP><<<grid, dim3(256), 0, s>>>(p);
+  if (BM == 128) {                 // 128 rows x 128 columns
+    dim3 grid((p.N + 127) / 128, max_tiles);
+    moe_gemm_kernel<4, 4, 2, UP><<<grid, dim3(256), 0, s>>>(p);
+  } else if (BM == 64) {           // 64 rows x 256 columns
+    dim3 grid((p.N + 255) / 256, max_tiles);
+    moe_gemm_kernel<4, 4, 1, UP><<<grid, dim3(256), 0, s>>>(p);
+  } else {                         // 16 rows x 128 columns
+    dim3 grid((p.N + 127) / 128, max_tiles);
+    moe_gemm_kernel<1, 2, 1, UP><<<grid, dim3(256), 0, s>>>(p);
   }
 }
 
@@ -185,7 +202,8 @@ extern "C" {
 
 int lv_moe_tile_rows(int64_t pairs, int E) {
   // few rows per expert (decoded tokens): tiles of 16 rows read each weight once and waste little of the matrix cores;
-  // prompts: 64 rows share every weight fragment
+  // prompts: 64 or 128 rows share every weight fragment
+  if (pairs >= static_cast<int64_t>(E) * 256) return 128;
   return pairs >= static_cast<int64_t>(E) * 48 ? 64 : 16;
 }
 

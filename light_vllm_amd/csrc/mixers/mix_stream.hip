@@ -125,32 +125,72 @@ static int hc_launch(void* x, const void* y, const void* mix, const void* out_w,
 
 // ------------------------------------------------------------------------------------------------
 // x f32 [T, W] += y1 + y2 (either may be absent); out = x / sqrt(mean(x^2) + eps) * (w_offset + w).
-template <typename T>
+// Four elements per thread and access (16-byte loads of the residual, 8-byte loads of bf16 rows) when W is a multiple of 4.
+__device__ __forceinline__ float4 ld4(const float* p) { return *reinterpret_cast<const float4*>(p); }
+__device__ __forceinline__ float4 ld4(const bf16_t* p) {
+  const uint2 v = *reinterpret_cast<const uint2*>(p);
+  return float4{__builtin_bit_cast(float, v.x << 16), __builtin_bit_cast(float, v.x & 0xffff0000u),
+                __builtin_bit_cast(float, v.y << 16), __builtin_bit_cast(float, v.y & 0xffff0000u)};
+}
+__device__ __forceinline__ void st4(float* p, float4 v) { *reinterpret_cast<float4*>(p) = v; }
+__device__ __forceinline__ void st4(bf16_t* p, float4 v) {
+  bf16_t a, b, c, d;
+  stf(&a, v.x); stf(&b, v.y); stf(&c, v.z); stf(&d, v.w);
+  *reinterpret_cast<uint2*>(p) = uint2{static_cast<uint32_t>(a.bits) | (static_cast<uint32_t>(b.bits) << 16),
+                                       static_cast<uint32_t>(c.bits) | (static_cast<uint32_t>(d.bits) << 16)};
+}
+
+template <typename T, int VEC>
 __global__ __launch_bounds__(256) void residual_add_norm_kernel(float* __restrict__ x, const T* __restrict__ y1,
                                                                  const T* __restrict__ y2, const float* __restrict__ w,
                                                                  float w_offset, T* __restrict__ out, int W, float eps) {
-  extern __shared__ float lds[];          // [W] the updated row, then [4] partial sums
+  extern __shared__ __attribute__((aligned(16))) float lds[];          // [W] the updated row, then [4] partial sums
   float* red = lds + W;
   const int64_t t = blockIdx.x;
   float* xt = x + t * W;
   float ss = 0.0f;
-  for (int i = threadIdx.x; i < W; i += blockDim.x) {
-    float v = xt[i];
-    if (y1 != nullptr || y2 != nullptr) {
-      float add = y1 != nullptr ? ldf(y1 + t * W + i) : 0.0f;
-      if (y2 != nullptr) add += ldf(y2 + t * W + i);
-      v += add;
-      xt[i] = v;
+  if (VEC == 4) {
+    for (int i = threadIdx.x * 4; i < W; i += blockDim.x * 4) {
+      float4 v = ld4(xt + i);
+      if (y1 != nullptr || y2 != nullptr) {
+        float4 add = y1 != nullptr ? ld4(y1 + t * W + i) : float4{0.0f, 0.0f, 0.0f, 0.0f};
+        if (y2 != nullptr) {
+          const float4 b = ld4(y2 + t * W + i);
+          add.x += b.x; add.y += b.y; add.z += b.z; add.w += b.w;
+        }
+        v.x += add.x; v.y += add.y; v.z += add.z; v.w += add.w;
+        st4(xt + i, v);
+      }
+      st4(lds + i, v);
+      ss += (v.x * v.x + v.y * v.y) + (v.z * v.z + v.w * v.w);
     }
-    lds[i] = v;
-    ss += v * v;
+  } else {
+    for (int i = threadIdx.x; i < W; i += blockDim.x) {
+      float v = xt[i];
+      if (y1 != nullptr || y2 != nullptr) {
+        float add = y1 != nullptr ? ldf(y1 + t * W + i) : 0.0f;
+        if (y2 != nullptr) add += ldf(y2 + t * W + i);
+        v += add;
+        xt[i] = v;
+      }
+      lds[i] = v;
+      ss += v * v;
+    }
   }
   if (out == nullptr) return;
   ss = wave_sum(ss);
   if (threadIdx.x % kWave == 0) red[threadIdx.x / kWave] = ss;
   __syncthreads();
   const float inv = 1.0f / sqrtf((red[0] + red[1] + red[2] + red[3]) / static_cast<float>(W) + eps);
-  for (int i = threadIdx.x; i < W; i += blockDim.x) stf(out + t * W + i, lds[i] * inv * (w_offset + w[i]));
+  if (VEC == 4) {
+    for (int i = threadIdx.x * 4; i < W; i += blockDim.x * 4) {       // each thread reads back what it wrote itself
+      const float4 v = ld4(lds + i), g = ld4(w + i);
+      st4(out + t * W + i, float4{v.x * inv * (w_offset + g.x), v.y * inv * (w_offset + g.y), v.z * inv * (w_offset + g.z),
+                                  v.w * inv * (w_offset + g.w)});
+    }
+  } else {
+    for (int i = threadIdx.x; i < W; i += blockDim.x) stf(out + t * W + i, lds[i] * inv * (w_offset + w[i]));
+  }
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -490,16 +530,20 @@ int lv_residual_add_norm(void* x, const void* y1, const void* y2, const void* w,
   const size_t shm = static_cast<size_t>(W + 4) * sizeof(float);
   if (shm > 64 * 1024) return fail(-2, "lv_residual_add_norm: width %d too large", W);
   dim3 grid(static_cast<unsigned>(T)), block(256);
-  if (dtype == LV_MIX_BF16)
-    residual_add_norm_kernel<bf16_t><<<grid, block, shm, as_stream(stream)>>>(
-        static_cast<float*>(x), static_cast<const bf16_t*>(y1), static_cast<const bf16_t*>(y2),
-        static_cast<const float*>(w), w_offset, static_cast<bf16_t*>(out), W, eps);
-  else if (dtype == LV_MIX_F32)
-    residual_add_norm_kernel<float><<<grid, block, shm, as_stream(stream)>>>(
-        static_cast<float*>(x), static_cast<const float*>(y1), static_cast<const float*>(y2),
-        static_cast<const float*>(w), w_offset, static_cast<float*>(out), W, eps);
-  else
+  auto aligned = [](const void* q) { return (reinterpret_cast<uintptr_t>(q) & 15) == 0; };
+  const bool vec = W % 4 == 0 && aligned(x) && aligned(y1) && aligned(y2) && aligned(w) && aligned(out);
+#define LVMIX_RES(TT, VV)                                                                                       \
+  residual_add_norm_kernel<TT, VV><<<grid, block, shm, as_stream(stream)>>>(                                   \
+      static_cast<float*>(x), static_cast<const TT*>(y1), static_cast<const TT*>(y2), static_cast<const float*>(w), \
+      w_offset, static_cast<TT*>(out), W, eps)
+  if (dtype == LV_MIX_BF16) {
+    if (vec) LVMIX_RES(bf16_t, 4); else LVMIX_RES(bf16_t, 1);
+  } else if (dtype == LV_MIX_F32) {
+    if (vec) LVMIX_RES(float, 4); else LVMIX_RES(float, 1);
+  } else {
     return fail(-1, "lv_residual_add_norm: dtype %d", dtype);
+  }
+#undef LVMIX_RES
   return launched("lv_residual_add_norm");
 }
 

@@ -20,7 +20,7 @@ def case_residual_norm(device, dtype):
     """One f32 residual: two sublayer outputs are added, the norm weight is applied as (offset + w)."""
     from light_vllm_amd import mix_ops
     g = torch.Generator().manual_seed(1)
-    for T, W in ((7, 48), (3, 40), (5, 1000)):
+    for T, W in ((7, 48), (3, 37), (5, 1000)):
         x = 5 * torch.randn(T, W, generator=g)
         y1, y2 = (torch.randn(T, W, generator=g).to(_dt(dtype)) for _ in range(2))
         w = 0.3 * torch.randn(W, generator=g)
@@ -320,7 +320,8 @@ def case_moe_ff(device, dtype):
     from light_vllm_amd.layers import moe as moe_mod
     g = torch.Generator().manual_seed(7)
     cases = [(24, 12, 6, 2, 3, 2, 19, "masked"), (64, 32, 8, 3, 4, 2, 1, "gathered"), (64, 32, 8, 3, 4, 2, 19, "gathered"),
-             (64, 32, 8, 3, 4, 2, 19, "masked"), (96, 64, 4, 1, 1, 1, 210, "gathered"), (32, 32, 16, 5, 1, 1, 333, "gathered")]
+             (64, 32, 8, 3, 4, 2, 19, "masked"), (96, 64, 4, 1, 1, 1, 210, "gathered"), (32, 32, 16, 5, 1, 1, 333, "gathered"),
+             (128, 64, 2, 1, 1, 1, 700, "gathered"), (192, 160, 3, 2, 1, 1, 500, "gathered"), (96, 96, 2, 2, 1, 1, 300, "gathered")]
     for (W, Fe, E, top, groups, keep, T, kernel) in cases:
         if kernel == "gathered" and dtype != "bfloat16" and device != "cpu":
             continue                                  # the gathered kernels are bf16 only
