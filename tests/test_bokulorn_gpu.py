@@ -64,6 +64,12 @@ def test_matrix_core_attention_agrees_with_the_vector_kernel(gpu, tmp_path):
         mix_ops.WINDOW_ATTN_KERNEL = old
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("seed", [101, 102, 103, 104])
+def test_engine_random_configs(gpu, tmp_path, seed, dtype):
+    C.case_engine_random_config(DEV, dtype, tmp_path, seed)
+
+
 def test_masked_experts_serve_the_model_like_the_gathered_ones(gpu, tmp_path):
     """The bf16 schedules above take the gathered form of the feed-forward (sizes in multiples of 32); here the
     masked form is forced on the same model."""
