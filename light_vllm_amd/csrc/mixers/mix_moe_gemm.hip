@@ -78,8 +78,10 @@ struct MoeGemmParams {
 
 // MB x NB blocks of 16 x 16 per wave; WM waves along the rows (1 or 2), the others along the columns: the workgroup's
 // tile is (16 MB WM) rows x (16 NB 4 / WM) columns. The fragments of the next 32-wide step over k are loaded before the
-// matrix instructions of the current one are issued, so that memory latency is covered by them.
-template <int MB, int NB, int WM, bool UP>
+// matrix instructions of the current one are issued, so that memory latency is covered by them. KU > 0 (tiles of a few
+// rows, where the weights are read once and the launch is bound by memory): the fragments of KU steps are requested
+// together instead, and many small workgroups keep the memory system full.
+template <int MB, int NB, int WM, bool UP, int KU = 0>
 __global__ __launch_bounds__(256) void moe_gemm_kernel(MoeGemmParams p) {
   const int tile = blockIdx.y, bx = blockIdx.x;
   if (tile >= p.num_tiles[0]) return;
@@ -122,13 +124,25 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(MoeGemmParams p) {
       for (int nb = 0; nb < NB; ++nb)
         acc[mb][nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(b[nb], a[mb], acc[mb][nb], 0, 0, 0);
   };
-  load(a0, b0, 0);
-  for (int k = 0; k < p.K; k += 64) {
-    if (k + 32 < p.K) load(a1, b1, k + 32);
-    multiply(a0, b0);
-    if (k + 32 >= p.K) break;
-    if (k + 64 < p.K) load(a0, b0, k + 64);
-    multiply(a1, b1);
+  if constexpr (KU > 0) {
+    bf16x8_t au[KU][MB], bu[KU][NB];
+    for (int k = 0; k < p.K; k += 32 * KU) {
+#pragma unroll
+      for (int u = 0; u < KU; ++u)
+        if (k + 32 * u < p.K) load(au[u], bu[u], k + 32 * u);
+#pragma unroll
+      for (int u = 0; u < KU; ++u)
+        if (k + 32 * u < p.K) multiply(au[u], bu[u]);
+    }
+  } else {
+    load(a0, b0, 0);
+    for (int k = 0; k < p.K; k += 64) {
+      if (k + 32 < p.K) load(a1, b1, k + 32);
+      multiply(a0, b0);
+      if (k + 32 >= p.K) break;
+      if (k + 64 < p.K) load(a0, b0, k + 64);
+      multiply(a1, b1);
+    }
   }
   // acc[mb][nb][i] = C[row = m0 + 16 mb + ln][n = n0 + 16 nb + 4 lg + i]
 #pragma unroll
@@ -188,9 +202,9 @@ static void gemm_launch(const MoeGemmParams& p, int max_tiles, int BM, hipStream
   } else if (BM == 64) {           // 64 rows x 256 columns
     dim3 grid((p.N + 255) / 256, max_tiles);
     moe_gemm_kernel<4, 4, 1, UP><<<grid, dim3(256), 0, s>>>(p);
-  } else {                         // 16 rows x 128 columns
-    dim3 grid((p.N + 127) / 128, max_tiles);
-    moe_gemm_kernel<1, 2, 1, UP><<<grid, dim3(256), 0, s>>>(p);
+  } else {                         // 16 rows x 64 columns, four steps over k requested at once
+    dim3 grid((p.N + 63) / 64, max_tiles);
+    moe_gemm_kernel<1, 1, 1, UP, 4><<<grid, dim3(256), 0, s>>>(p);
   }
 }
 
