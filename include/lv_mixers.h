@@ -179,6 +179,16 @@ int lv_moe_grouped_ff(const void* h, const void* ids, const void* weights, const
                       void* workspace, int64_t T, int W, int F, int E, int top, void* stream);
 int64_t lv_moe_grouped_workspace_bytes(int64_t T, int W, int F, int E, int top);
 
+/* The sort and the weighted sum of the gathered form on their own, for callers that multiply the sorted rows themselves.
+ * ids int32 [M] (expert of pair p = token * top + choice) -> sorted_pair int32 (pair of each row in expert order),
+ * inv int32 [M] (row of each pair), offsets int32 [E + 1] (first row of each expert). Every expert's rows start on a
+ * multiple of `align`, so an expert owns rows [offsets[e], offsets[e + 1]), the last ones of which may be padding that the
+ * kernel does not write: sorted_pair has room for M + E * align entries and is cleared by the caller. */
+int lv_moe_sort(const void* ids, int64_t M, int E, int align, void* sorted_pair, void* inv, void* offsets, void* stream);
+/* rows bf16 [M, W] (expert outputs in sorted order), inv int32 [T, top], weights f32 [T, top]:
+ * out bf16 [T, W] = sum_k weights[t, k] * rows[inv[t, k]] in f32; W a multiple of 4. */
+int lv_moe_combine(const void* rows, const void* inv, const void* weights, void* out, int64_t T, int W, int top, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

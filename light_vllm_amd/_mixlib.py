@@ -48,6 +48,8 @@ SIGNATURES = {
     "lv_relu2_scale": (c_int, [_P, _P, _P, c_int64, c_int, c_int, c_int, _P]),
     "lv_moe_grouped_ff": (c_int, [_P, _P, _P, _P, _P, _P, _P, c_int64, c_int, c_int, c_int, c_int, _P]),
     "lv_moe_grouped_workspace_bytes": (c_int64, [c_int64, c_int, c_int, c_int, c_int]),
+    "lv_moe_sort": (c_int, [_P, c_int64, c_int, c_int, _P, _P, _P, _P]),
+    "lv_moe_combine": (c_int, [_P, _P, _P, _P, c_int64, c_int, c_int, _P]),
 }
 
 _lib = None

@@ -15,6 +15,8 @@
 //   moe_combine_kernel   one workgroup per token: sum over its choices of weight * expert output row, in f32.
 // A row's result does not depend on where the sort put it or on what else is in the tile: every output element is
 // its own chain of MFMA accumulations over k.
+// lv_moe_sort and lv_moe_combine are also exported alone: large eager steps run the experts' products as vendor GEMMs
+// on the sorted rows in between (mix_ops.moe_sorted_ff).
 #include "mix_common.h"
 
 namespace lvmix {
@@ -29,7 +31,7 @@ constexpr int kSortThreads = 1024;
 __global__ __launch_bounds__(kSortThreads) void moe_sort_kernel(const int32_t* __restrict__ ids, int M, int E, int BM,
                                                                  int32_t* __restrict__ sorted_pair, int32_t* __restrict__ inv,
                                                                  int32_t* __restrict__ tiles, int32_t* __restrict__ num_tiles,
-                                                                 int max_tiles) {
+                                                                 int max_tiles, int32_t* __restrict__ offsets, int align) {
   extern __shared__ int32_t sl[];
   int32_t* cnt = sl;              // [E] pairs per expert
   int32_t* off = sl + E;          // [E + 1] first row per expert
@@ -43,19 +45,22 @@ __global__ __launch_bounds__(kSortThreads) void moe_sort_kernel(const int32_t* _
     for (int e = 0; e < E; ++e) {
       off[e] = r;
       toff[e] = t;
-      r += cnt[e];
+      r = (r + cnt[e] + align - 1) / align * align;           // every expert starts on a multiple of `align` rows
       t += (cnt[e] + BM - 1) / BM;
     }
     off[E] = r;
     toff[E] = t;
-    num_tiles[0] = t < max_tiles ? t : max_tiles;
+    if (num_tiles != nullptr) num_tiles[0] = t < max_tiles ? t : max_tiles;
   }
   __syncthreads();
+  if (offsets != nullptr)
+    for (int e = threadIdx.x; e <= E; e += blockDim.x) offsets[e] = off[e];
   for (int p = threadIdx.x; p < M; p += blockDim.x) {
     const int row = off[ids[p]] + inv[p];
     sorted_pair[row] = p;
     inv[p] = row;
   }
+  if (tiles == nullptr) return;
   for (int e = threadIdx.x; e < E; e += blockDim.x) {
     const int n = cnt[e];
     for (int j = 0, t = toff[e]; j * BM < n && t < max_tiles; ++j, ++t) {
@@ -249,7 +254,7 @@ int lv_moe_grouped_ff(const void* h, const void* ids, const void* weights, const
   hipStream_t s = as_stream(stream);
   const size_t shm = sizeof(int32_t) * (3 * static_cast<size_t>(E) + 2);
   moe_sort_kernel<<<dim3(1), dim3(kSortThreads), shm, s>>>(static_cast<const int32_t*>(ids), static_cast<int>(M), E, BM,
-                                                          sorted_pair, inv, tiles, num_tiles, max_tiles);
+                                                          sorted_pair, inv, tiles, num_tiles, max_tiles, nullptr, 1);
   MoeGemmParams up{static_cast<const uint16_t*>(h), static_cast<const uint16_t*>(up_w), act, sorted_pair, tiles, num_tiles,
                    F, W, top, W, W, F, static_cast<int64_t>(F) * W};
   gemm_launch<true>(up, max_tiles, BM, s);
@@ -259,6 +264,26 @@ int lv_moe_grouped_ff(const void* h, const void* ids, const void* weights, const
   moe_combine_kernel<<<dim3(static_cast<unsigned>(T)), dim3(256), 0, s>>>(rows, inv, static_cast<const float*>(weights),
                                                                           static_cast<uint16_t*>(out), W, top);
   return launched("lv_moe_grouped_ff");
+}
+
+int lv_moe_sort(const void* ids, int64_t M, int E, int align, void* sorted_pair, void* inv, void* offsets, void* stream) {
+  if (M == 0) return 0;
+  if (!ids || !sorted_pair || !inv || !offsets || M < 0 || M > (1 << 29) || E <= 0 || E > 4096 || align <= 0 || align > 4096)
+    return fail(-1, "lv_moe_sort: bad arguments");
+  const size_t shm = sizeof(int32_t) * (3 * static_cast<size_t>(E) + 2);
+  moe_sort_kernel<<<dim3(1), dim3(kSortThreads), shm, as_stream(stream)>>>(
+      static_cast<const int32_t*>(ids), static_cast<int>(M), E, 1 << 30, static_cast<int32_t*>(sorted_pair),
+      static_cast<int32_t*>(inv), nullptr, nullptr, 0, static_cast<int32_t*>(offsets), align);
+  return launched("lv_moe_sort");
+}
+
+int lv_moe_combine(const void* rows, const void* inv, const void* weights, void* out, int64_t T, int W, int top, void* stream) {
+  if (T == 0) return 0;
+  if (!rows || !inv || !weights || !out || T < 0 || W <= 0 || W % 4 != 0 || top <= 0) return fail(-1, "lv_moe_combine: bad arguments");
+  moe_combine_kernel<<<dim3(static_cast<unsigned>(T)), dim3(256), 0, as_stream(stream)>>>(
+      static_cast<const uint16_t*>(rows), static_cast<const int32_t*>(inv), static_cast<const float*>(weights),
+      static_cast<uint16_t*>(out), W, top);
+  return launched("lv_moe_combine");
 }
 
 int64_t lv_moe_grouped_workspace_bytes(int64_t T, int W, int F, int E, int top) {

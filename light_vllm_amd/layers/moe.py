@@ -12,12 +12,16 @@ matrices one [width, experts * ff] weight. Two forms compute the same sum:
   * gathered (bf16, width and ff in multiples of 32, at least GATHER_FROM experts per choice): the (token,
     choice) pairs are sorted by expert on the device and every expert multiplies only its own rows
     (mix_ops.moe_grouped_ff: sort, two grouped GEMMs on the matrix cores, weighted sum; four launches);
+  * sorted (bf16, eager steps with at least SORTED_FROM rows per expert): the same device-side sort, then every
+    expert's two products as vendor GEMMs on its slice of the sorted rows, after reading the experts' row counts
+    back once (mix_ops.moe_sorted_ff); large prompt steps, where the vendor GEMM's rate outweighs the one host
+    synchronisation. Steps captured into a hipGraph never take it;
   * masked (f32, other sizes, few experts per choice): the up projection of every expert in one vendor
     GEMM, one kernel applies the activation times the token's weight for the column's expert (zero for
     experts the token did not choose), and the down GEMM sums over experts by itself. It spends
     experts / top times the FLOPs of the gathered form.
 
-Neither synchronises with the host, so both can be captured into a hipGraph.
+The gathered and masked forms never synchronise with the host, so both can be captured into a hipGraph.
 """
 from __future__ import annotations
 
@@ -26,11 +30,13 @@ import torch.nn.functional as F
 from torch import nn
 
 from .. import mix_ops
+from ..utils.context import get_context
 from .tp import tp_size
 
 
 GATHER_FROM = 2.0     # experts / top from which the gathered form is taken
-MOE_KERNEL = "auto"   # "auto" | "masked" | "gathered" (tests force one or the other)
+SORTED_FROM = 256     # rows per expert from which an eager step runs the experts as vendor GEMMs on sorted rows
+MOE_KERNEL = "auto"   # "auto" | "masked" | "gathered" | "sorted" (tests force one or the other)
 
 
 class SparseMoE(nn.Module):
@@ -56,14 +62,21 @@ class SparseMoE(nn.Module):
         logits = F.linear(h.float(), self.router_weight)
         return mix_ops.moe_route(logits, self.correction, self.top, self.groups, self.keep)
 
-    def gathered(self, h: torch.Tensor) -> bool:
+    def form(self, h: torch.Tensor) -> str:
         if MOE_KERNEL != "auto":
-            return MOE_KERNEL == "gathered"
-        return mix_ops.moe_grouped_ok(h, self.ff) and self.E >= GATHER_FROM * self.top
+            return MOE_KERNEL
+        if not (mix_ops.moe_grouped_ok(h, self.ff) and self.E >= GATHER_FROM * self.top):
+            return "masked"
+        step = get_context().ragged
+        captured = step is not None and step.static
+        return "sorted" if not captured and h.size(0) * self.top >= SORTED_FROM * self.E else "gathered"
 
     def forward(self, h: torch.Tensor) -> torch.Tensor:
         ids, weights, dense = self.route(h)
-        if self.gathered(h):
+        form = self.form(h)
+        if form == "gathered":
             return mix_ops.moe_grouped_ff(h, ids, weights, self.up_weight, self.down_weight, self.E, self.ff)
+        if form == "sorted":
+            return mix_ops.moe_sorted_ff(h, ids, weights, self.up_weight, self.down_weight, self.E, self.ff)
         up = F.linear(h, self.up_weight)
         return F.linear(mix_ops.relu2_scale(up, dense, self.E, self.ff), self.down_weight)

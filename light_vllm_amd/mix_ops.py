@@ -554,3 +554,70 @@ def moe_grouped_ff(h, ids, weights, up_w, down_w, E, Fe):
         acc.index_add_(0, t_idx, y * weights[t_idx, k_idx][:, None])
     out.copy_(acc)
     return out
+
+
+def moe_sort(ids, E, align=1):
+    """ids int32 [T, top] -> (sorted_pair [M + E * align], inv [T, top], offsets [E + 1]), int32: the (token, choice)
+    pairs in expert order, the row each pair got, and the first row of every expert. Every expert starts on a multiple
+    of `align` rows: expert e owns rows offsets[e] .. offsets[e + 1], the last of which may be padding (pair 0)."""
+    M = ids.numel()
+    dev = ids.device
+    if ids.is_cuda:
+        sorted_pair = torch.zeros(M + E * align, dtype=torch.int32, device=dev)
+        inv = torch.empty_like(ids)
+        offsets = torch.empty(E + 1, dtype=torch.int32, device=dev)
+        lib = _mixlib.load()
+        _mixlib.check(lib.lv_moe_sort(_p(ids), M, E, align, _p(sorted_pair), _p(inv), _p(offsets), _stream(ids)), "lv_moe_sort")
+        return sorted_pair, inv, offsets
+    flat = ids.reshape(-1).long()
+    order = torch.sort(flat, stable=True).indices
+    counts = torch.bincount(flat, minlength=E)
+    padded = (counts + align - 1) // align * align
+    offsets = torch.cat([torch.zeros(1, dtype=torch.long), padded.cumsum(0)])
+    rank = torch.arange(M) - (counts.cumsum(0) - counts)[flat[order]]
+    rows = offsets[flat[order]] + rank
+    sorted_pair = torch.zeros(M + E * align, dtype=torch.int32)
+    sorted_pair[rows] = order.to(torch.int32)
+    inv = torch.empty(M, dtype=torch.int32)
+    inv[order] = rows.to(torch.int32)
+    return sorted_pair, inv.view_as(ids), offsets.to(torch.int32)
+
+
+def moe_combine(rows, inv, weights):
+    """rows act [M, W] (expert outputs in sorted order) -> act [T, W] = sum_k weights[t, k] * rows[inv[t, k]], in f32."""
+    T, top = inv.shape
+    W = rows.size(1)
+    out = torch.empty(T, W, dtype=rows.dtype, device=rows.device)
+    if rows.is_cuda:
+        assert rows.dtype == torch.bfloat16 and rows.is_contiguous() and W % 4 == 0 and weights.dtype == torch.float32
+        lib = _mixlib.load()
+        _mixlib.check(lib.lv_moe_combine(_p(rows), _p(inv), _p(weights), _p(out), T, W, top, _stream(rows)), "lv_moe_combine")
+        return out
+    out.copy_((rows[inv.long()].float() * weights[:, :, None]).sum(1))
+    return out
+
+
+SORTED_ALIGN = 128
+
+
+def moe_sorted_ff(h, ids, weights, up_w, down_w, E, Fe):
+    """The same sum as moe_grouped_ff for large eager steps: rows sorted by expert on the device, the experts' row
+    counts read back once, and each expert's two products run as vendor GEMMs on its slice of the sorted rows. One host
+    synchronisation per call, so not for steps that are captured into a graph. Every expert's slice is padded to a
+    multiple of SORTED_ALIGN rows (copies of token 0 that no one reads back): the GEMM library then sees a handful of
+    shapes instead of a new one per expert and step, each of which would cost it a kernel selection on the host."""
+    T, W = h.shape
+    top = ids.size(1)
+    sorted_pair, inv, offsets = moe_sort(ids, E, SORTED_ALIGN)
+    off = offsets.tolist()
+    xs = h.index_select(0, torch.div(sorted_pair[:off[E]], top, rounding_mode="floor"))
+    act = torch.empty(off[E], Fe, dtype=h.dtype, device=h.device)
+    for e in range(E):
+        if off[e + 1] > off[e]:
+            torch.mm(xs[off[e]:off[e + 1]], up_w[e * Fe:(e + 1) * Fe].t(), out=act[off[e]:off[e + 1]])
+    act.relu_().square_()
+    rows = torch.empty(off[E], W, dtype=h.dtype, device=h.device)
+    for e in range(E):
+        if off[e + 1] > off[e]:
+            torch.mm(act[off[e]:off[e + 1]], down_w[:, e * Fe:(e + 1) * Fe].t(), out=rows[off[e]:off[e + 1]])
+    return moe_combine(rows, inv, weights)

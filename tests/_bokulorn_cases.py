@@ -321,9 +321,10 @@ def case_moe_ff(device, dtype):
     g = torch.Generator().manual_seed(7)
     cases = [(24, 12, 6, 2, 3, 2, 19, "masked"), (64, 32, 8, 3, 4, 2, 1, "gathered"), (64, 32, 8, 3, 4, 2, 19, "gathered"),
              (64, 32, 8, 3, 4, 2, 19, "masked"), (96, 64, 4, 1, 1, 1, 210, "gathered"), (32, 32, 16, 5, 1, 1, 333, "gathered"),
-             (128, 64, 2, 1, 1, 1, 700, "gathered"), (192, 160, 3, 2, 1, 1, 500, "gathered"), (96, 96, 2, 2, 1, 1, 300, "gathered")]
+             (128, 64, 2, 1, 1, 1, 700, "gathered"), (192, 160, 3, 2, 1, 1, 500, "gathered"), (96, 96, 2, 2, 1, 1, 300, "gathered"),
+             (64, 32, 8, 3, 4, 2, 19, "sorted"), (192, 160, 3, 2, 1, 1, 500, "sorted"), (32, 32, 16, 5, 1, 1, 333, "sorted")]
     for (W, Fe, E, top, groups, keep, T, kernel) in cases:
-        if kernel == "gathered" and dtype != "bfloat16" and device != "cpu":
+        if kernel in ("gathered", "sorted") and dtype != "bfloat16" and device != "cpu":
             continue                                  # the gathered kernels are bf16 only
         mlp = {"expert": {"ff": Fe}, "router": {"experts": E, "top": top, "groups": {"count": groups, "keep": keep}}}
         weights = {"router": 2 * torch.randn(E, W, generator=g) / W ** 0.5, "correction": 0.3 * torch.randn(E, generator=g)}
@@ -496,3 +497,34 @@ def case_generate(device, tmp_path, enforce_eager=True):
             assert (top2[0] - top2[1]).item() > 2e-4 * logits.abs().max().item(), "oracle tie: pick another seed"
             seq.append(int(logits.argmax()))
         assert out["token_ids"] == seq[len(p):]
+
+
+def case_generate_bf16_graphs_like_eager(device, tmp_path):
+    """bf16, sizes that take the matrix-core attention and the gathered experts: single-token steps replayed from
+    hipGraphs (launch geometry fixed at its bound, padded rows) continue every prompt like eager steps do, wherever
+    the oracle's choice of the next token is no close call."""
+    from light_vllm_amd.llm import LLM
+    from light_vllm_amd.sampling_params import SamplingParams
+    cfg = K.CFG_WIDE
+    model_dir, weights = _model(tmp_path, cfg, 12)
+    prompts = [K.tokens_for(cfg, n, 70 + n) for n in (40, 9, 23)]
+    steps = 8
+    outs = {}
+    for eager in (True, False):
+        llm = LLM(model_dir, dtype="bfloat16", device=device, kvcache_block_size=16, max_num_seqs=4, max_cache_tokens=256,
+                  max_num_batched_tokens=64, max_model_len=64, enforce_eager=eager)
+        outs[eager] = [o["token_ids"] for o in llm.generate([list(p) for p in prompts],
+                                                           SamplingParams(temperature=0.0, max_tokens=steps, ignore_eos=True))]
+        llm.exit()
+    compared = 0
+    for p, a, b in zip(prompts, outs[True], outs[False]):
+        seq = list(p)
+        for x, y in zip(a, b):
+            logits = oracle.forward(cfg, weights, seq)[-1]
+            top2 = logits.topk(2).values
+            if (top2[0] - top2[1]).item() < 0.05 * logits.std().item() or x != int(logits.argmax()):
+                break                       # a close call (or bf16 already chose otherwise): the continuations part ways
+            assert x == y, (seq[len(p):], a, b)
+            compared += 1
+            seq.append(x)
+    assert compared >= steps, "too few decided tokens: pick another seed"

@@ -81,6 +81,16 @@ def test_masked_experts_serve_the_model_like_the_gathered_ones(gpu, tmp_path):
         moe.MOE_KERNEL = old
 
 
+def test_sorted_experts_serve_the_model_like_the_gathered_ones(gpu, tmp_path):
+    """The form that large eager steps take (vendor GEMMs on rows sorted by expert), forced on the same small model."""
+    from light_vllm_amd.layers import moe
+    old, moe.MOE_KERNEL = moe.MOE_KERNEL, "sorted"
+    try:
+        C.case_engine_schedules(DEV, "bfloat16", tmp_path, cfg=K.CFG_WIDE, seed=11)
+    finally:
+        moe.MOE_KERNEL = old
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_engine_reuse_of_pages_and_slots(gpu, tmp_path, dtype):
     C.case_engine_reuse(DEV, dtype, tmp_path)
@@ -98,3 +108,7 @@ def test_generate_greedy_from_graphs(gpu, tmp_path):
     """Steps of single tokens replay captured hipGraphs (padded rows included, many replays between eager prompt
     steps): the completions are the oracle's all the same."""
     C.case_generate(DEV, tmp_path, enforce_eager=False)
+
+
+def test_generate_bf16_from_graphs_like_eager(gpu, tmp_path):
+    C.case_generate_bf16_graphs_like_eager(DEV, tmp_path)
