@@ -24,6 +24,7 @@
  *   lv_moe_route             sigmoid router with a selection-only correction, group limit and top-k
  *   lv_relu2_scale           squared relu of the experts' up projections times the routing weight
  *   lv_moe_grouped_ff        the experts' feed-forward on rows sorted by expert (grouped GEMMs on the matrix cores)
+ *   lv_moe_sort, lv_moe_combine   its first and last step alone, for callers that multiply the sorted rows themselves
  *
  * A "ragged step" is a batch of B sequences; sequence b brings cu_q[b+1]-cu_q[b] new tokens that
  * follow ctx_lens[b] tokens already in the cache / state (a whole prompt, a portion of one, or one
