@@ -4,7 +4,7 @@
 //                             projection (before they are split into heads), K and V rows scattered into the cache.
 //   pool_update_kernel        one workgroup per (sequence, block completed by this step): mean of its P cached
 //                             keys and values, stored with the page of the block's last token.
-//   window_pool_attn_kernel   one workgroup per (token, kv head, group of up to 8 query heads). The key list of a
+//   window_pool_attn_kernel   one workgroup per (token, kv head, group of up to 8 query heads; 4 for value sizes above 256). The key list of a
 //                             query is [pooled blocks wholly before the window | tokens of the window]; the four
 //                             waves take 64-key chunks in turn (lane = key for the scores, lane = value column
 //                             for the weighted sum), each with its own running maximum, and merge in LDS. The
@@ -87,10 +87,9 @@ struct WindowAttnParams {
   float m0;             // where the running maximum starts: the sink's score 0, or far below any score without a sink
 };
 
-constexpr int kMaxRep = 8;      // query heads of one kv head served by one workgroup
-constexpr int kMaxDvi = 4;      // value columns per lane: Dv <= 256
-
-template <typename T>
+// kMaxRep: query heads of one kv head served by one workgroup; kMaxDvi: value columns per lane (Dv <= 64 * kMaxDvi).
+// Instantiated for (8, 4): value sizes up to 256, and (4, 8): up to 512 with half the heads per workgroup.
+template <typename T, int kMaxRep, int kMaxDvi>
 __global__ __launch_bounds__(256) void window_pool_attn_kernel(WindowAttnParams p) {
   extern __shared__ float lds[];
   const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
@@ -298,7 +297,9 @@ int lv_window_pool_attn(const void* q, const void* k_cache, const void* v_cache,
   if (P > 0 && (!kp || !vp)) return fail(-1, "lv_window_pool_attn: pooled blocks without their cache");
   if (T < 0 || H <= 0 || G <= 0 || H % G != 0 || D <= 0 || Dv <= 0 || page <= 0 || window <= 0 || bt_stride <= 0)
     return fail(-1, "lv_window_pool_attn: bad sizes");
-  if (Dv > kMaxDvi * kWave) return fail(-2, "lv_window_pool_attn: value size %d above %d", Dv, kMaxDvi * kWave);
+  if (Dv > 8 * kWave) return fail(-2, "lv_window_pool_attn: value size %d above %d", Dv, 8 * kWave);
+  const bool wide = Dv > 4 * kWave;
+  const int kMaxRep = wide ? 4 : 8;
   const int rep = H / G;
   WindowAttnParams p{q, k_cache, v_cache, kp, vp, gate, ld_gate, out, cu_q, ctx_lens, tok_seq, block_tables,
                      bt_stride, H, G, D, Dv, page, window, P, P > 0 ? (page + P - 1) / P : 0, scale,
@@ -307,9 +308,14 @@ int lv_window_pool_attn(const void* q, const void* k_cache, const void* v_cache,
                                       4 * static_cast<size_t>(kMaxRep) * Dv + 4 * kMaxRep * 2);
   if (shm > 64 * 1024) return fail(-2, "lv_window_pool_attn: head sizes %d / %d need %zu bytes of LDS", D, Dv, shm);
   dim3 grid(static_cast<unsigned>(T), G, (rep + kMaxRep - 1) / kMaxRep), block(256);
-  if (dtype == LV_MIX_BF16) window_pool_attn_kernel<bf16_t><<<grid, block, shm, as_stream(stream)>>>(p);
-  else if (dtype == LV_MIX_F32) window_pool_attn_kernel<float><<<grid, block, shm, as_stream(stream)>>>(p);
-  else return fail(-1, "lv_window_pool_attn: dtype %d", dtype);
+  if (dtype != LV_MIX_BF16 && dtype != LV_MIX_F32) return fail(-1, "lv_window_pool_attn: dtype %d", dtype);
+  if (dtype == LV_MIX_BF16) {
+    if (wide) window_pool_attn_kernel<bf16_t, 4, 8><<<grid, block, shm, as_stream(stream)>>>(p);
+    else window_pool_attn_kernel<bf16_t, 8, 4><<<grid, block, shm, as_stream(stream)>>>(p);
+  } else {
+    if (wide) window_pool_attn_kernel<float, 4, 8><<<grid, block, shm, as_stream(stream)>>>(p);
+    else window_pool_attn_kernel<float, 8, 4><<<grid, block, shm, as_stream(stream)>>>(p);
+  }
   return launched("lv_window_pool_attn");
 }
 

@@ -101,7 +101,8 @@ def case_latent_attention_beacons(device, dtype):
     from light_vllm_amd import mix_ops
     from light_vllm_amd.layers.latent_attention import NO_WINDOW
     for (H, R, Dr, page, L) in ((3, 24, 8, 16, 300), (1, 70, 6, 64, 333), (10, 9, 0, 16, 120),
-                                (5, 32, 16, 16, 300), (4, 64, 0, 32, 410), (2, 160, 32, 64, 200)):
+                                (5, 32, 16, 16, 300), (4, 64, 0, 32, 410), (2, 160, 32, 64, 200),
+                                (5, 320, 32, 64, 150)):              # a latent above 256: the vector kernel with four heads a workgroup
         beacons = [0, 1, page - 1, page, 2 * page + 1, 50]
         rows, e, table, cache = _latent_rows(L, R, Dr, page, L + H, dtype, device, beacons)
         g = torch.Generator().manual_seed(L)
